@@ -17,7 +17,7 @@ import numpy as np
 
 # ----------------------------------------------------------------------------- files
 def read_safetensors(path):
-    """name -> float64 array (bf16/f16/f32 widened exactly)."""
+    """name -> float64 array (bf16/f16/f32 widened exactly; integer tensors as int64)."""
     with open(path, "rb") as f:
         (n,) = struct.unpack("<Q", f.read(8))
         header = json.loads(f.read(n).decode("utf-8"))
@@ -36,6 +36,8 @@ def read_safetensors(path):
             arr = np.frombuffer(raw, dtype="<f4").astype(np.float64)
         elif dt == "F16":
             arr = np.frombuffer(raw, dtype="<f2").astype(np.float64)
+        elif dt in ("I32", "I64"):          # integer tables stay integers
+            arr = np.frombuffer(raw, dtype="<i4" if dt == "I32" else "<i8").astype(np.int64)
         else:
             raise ValueError(f"{name}: dtype {dt}")
         out[name] = arr.reshape(info["shape"])
@@ -82,6 +84,8 @@ class TensorsOnDemand:
             arr = np.frombuffer(raw, dtype="<f4").astype(np.float64)
         elif dt == "F16":
             arr = np.frombuffer(raw, dtype="<f2").astype(np.float64)
+        elif dt in ("I32", "I64"):          # integer tables stay integers
+            arr = np.frombuffer(raw, dtype="<i4" if dt == "I32" else "<i8").astype(np.int64)
         else:
             raise ValueError(f"{name}: dtype {dt}")
         return arr.reshape(info["shape"])

@@ -41,6 +41,7 @@ class LayerSpec:
     feed_forward: Optional[PartSpec] = None
     norms: Mapping[str, PartSpec] = field(default_factory=dict)
     block: str = "prenorm"
+    block_params: Mapping[str, Any] = field(default_factory=dict)        # constants of the arrangement itself (a factor on what a sublayer adds, say)
     filters: Mapping[str, PartSpec] = field(default_factory=dict)    # sequence filters, by the arrangement's names
     connections: Mapping[str, PartSpec] = field(default_factory=dict)    # how sublayers meet the residual streams, likewise
 
@@ -53,9 +54,12 @@ class ExecStep:
     entries: its weights are shared, each entry has a cache of its own).
     ``cache_of`` is the index of an earlier entry whose cache this entry reads
     instead of owning one; such an entry writes no keys or values.
+    ``enters``: the model's ``injection`` runs right before this entry (the first layer of a pass
+    over a looped span, say).
     """
     layer: int
     cache_of: Optional[int] = None
+    enters: bool = False
 
 
 @dataclass(frozen=True)
@@ -72,11 +76,16 @@ class ModelSpec:
     eos_token_ids: tuple = ()
     bos_token_id: Optional[int] = None
     streams: Optional[int] = None       # copies of the residual stream the layers keep (None: the one stream)
+    injection: Optional[PartSpec] = None    # what remakes the residual stream from itself and the embedding's rows before the entries that say ``enters``
 
     def validate(self) -> None:
         if self.streams is not None and self.streams < 1:
             raise ValueError(f"a model has at least one residual stream, not {self.streams}")
+        if self.injection is not None and self.streams is not None:
+            raise ValueError("an injection of the embedding's rows is built for the one residual stream")
         for i, st in enumerate(self.order):
+            if st.enters and self.injection is None:
+                raise ValueError(f"run order entry {i} is entered through an injection the model does not have")
             if not (0 <= st.layer < len(self.layers)):
                 raise ValueError(f"run order entry {i} names layer {st.layer}, model has {len(self.layers)}")
             if st.cache_of is not None:

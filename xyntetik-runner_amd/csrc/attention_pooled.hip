@@ -63,6 +63,46 @@ extern "C" int xr_qkv_store(void* q_out, void* k_cache, void* v_cache, const flo
     return XR_OK;
 }
 
+// ---------------------------------------------------------------- a norm of every query and key head
+// In place on the 32-bit projections, between the product and the store: every head of D channels is divided
+// by its root mean square (eps inside the root) and multiplied by a weight over D that the heads share (one for
+// the queries, one for the keys; either may be absent: that side is left alone).  With `every` > 0 the queries
+// of the token at position p are also multiplied by 1 + coef * ln(floor((p + 1) / every) + 1): queries far
+// into a sequence are sharpened.  A wave a head.
+__global__ __launch_bounds__(256) void k_head_rmsnorm(float* __restrict__ q, float* __restrict__ k, int ld,
+                                                      const float* __restrict__ wq, const float* __restrict__ wk,
+                                                      const int* __restrict__ positions, int H, int Hk, int D, float eps,
+                                                      float coef, int every) {
+    const int t = blockIdx.x, lane = threadIdx.x & 63;
+    const int head = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (head >= H + Hk) return;
+    const bool is_q = head < H;
+    const float* w = is_q ? wq : wk;
+    float temp = 1.f;
+    if (is_q && every > 0) temp = 1.0f + coef * logf((float)((positions[t] + 1) / every + 1));
+    if (!w && temp == 1.f) return;
+    float* x = (is_q ? q + (size_t)head * D : k + (size_t)(head - H) * D) + (size_t)t * ld;
+    float f = temp;
+    if (w) {
+        float ss = 0.f;
+        for (int d = lane; d < D; d += 64) ss = fmaf(x[d], x[d], ss);
+        f *= 1.0f / sqrtf(wave_sum(ss) / (float)D + eps);
+    }
+    for (int d = lane; d < D; d += 64) x[d] = x[d] * f * (w ? w[d] : 1.f);
+}
+
+extern "C" int xr_head_rmsnorm(float* q, float* k, int ld, const float* wq, const float* wk, const int* positions, int T,
+                               int H, int Hk, int D, float eps, float coef, int every, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && H >= 0 && Hk >= 0 && D > 0, "head_rmsnorm: bad sizes T=%d H=%d Hk=%d D=%d", T, H, Hk, D);
+    XR_REQUIRE((H == 0 || q) && (Hk == 0 || k), "head_rmsnorm: heads without their rows");
+    XR_REQUIRE(every >= 0 && (every == 0 || positions), "head_rmsnorm: a temperature every %d positions needs the positions", every);
+    XR_REQUIRE(eps >= 0.f, "head_rmsnorm: eps %g is negative", eps);
+    if (T == 0 || H + Hk == 0) return XR_OK;
+    k_head_rmsnorm<<<dim3(T, (H + Hk + 3) / 4), 256, 0, stream>>>(q, k, ld, wq, wk, positions, H, Hk, D, eps, coef, every);
+    XR_CHECK_LAUNCH("head_rmsnorm");
+    return XR_OK;
+}
+
 // ---------------------------------------------------------------- the means of the blocks a step completes
 // Request b held starts[b] positions before the step and brings n = cu_q[b+1] - cu_q[b]: the
 // blocks starts[b] / P .. (starts[b] + n) / P - 1 are complete now.  One workgroup per

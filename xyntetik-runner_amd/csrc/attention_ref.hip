@@ -8,7 +8,8 @@
 // (src/model.c:3553-3573, :6326); softmax with the maximum taken out
 // (src/model.c:3409-3415); out = sum_t p_t V_t (:3576-3587).  The
 // softmax runs over blocks of 64 keys with a running maximum and sum, which gives the
-// same value up to rounding.
+// same value up to rounding.  With `slopes` (one number a query head) a bias that grows with the distance is
+// taken off every score: s_t = (q . K_t) * scale - slope_h * (p - t).
 #include "common.h"
 
 #define AR_MAX_D 256
@@ -18,7 +19,7 @@ __global__ __launch_bounds__(64) void k_attention_ref(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
     const int* __restrict__ block_table, int table_stride, int H, int Hk, int D, int page_shift,
-    int page_mask, int page_size, float scale, int window) {
+    int page_mask, int page_size, float scale, int window, const float* __restrict__ slopes) {
     __shared__ float qs[AR_MAX_D];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
@@ -29,6 +30,7 @@ __global__ __launch_bounds__(64) void k_attention_ref(
     for (int d = lane; d < D; d += 64) qs[d] = ld<T>(qrow, d);
     __syncthreads();
     const int* bt = block_table + (size_t)req * table_stride;
+    const float slope = slopes ? slopes[h] : 0.f;
 
     float m = -INFINITY, l = 0.f;
     float acc[AR_MAX_D / 64];
@@ -45,7 +47,7 @@ __global__ __launch_bounds__(64) void k_attention_ref(
             const T* kr = kc + (((size_t)page * Hk + kvh) * page_size + off) * D;
             float dot = 0.f;
             for (int d = 0; d < D; ++d) dot = fmaf(qs[d], ld<T>(kr, d), dot);
-            s = dot * scale;
+            s = dot * scale - slope * (float)(pos - key);
         }
         const float mn = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - mn) : 0.f;
@@ -79,7 +81,7 @@ __global__ __launch_bounds__(64) void k_attention_ref(
 extern "C" int xr_attention_ref(void* out, const void* q, const void* k_cache, const void* v_cache,
                                 const int* positions, const int* req_of_token, const int* block_table,
                                 int table_stride, int T, int H, int Hk, int D, int page_size, float scale,
-                                int window, int dtype, hipStream_t stream) {
+                                int window, int dtype, const float* slopes, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && H > 0 && Hk > 0 && D > 0, "attention: bad sizes T=%d H=%d Hk=%d D=%d", T, H, Hk, D);
     XR_REQUIRE(H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
     XR_REQUIRE(D <= AR_MAX_D, "attention: head size %d exceeds %d", D, AR_MAX_D);
@@ -91,11 +93,11 @@ extern "C" int xr_attention_ref(void* out, const void* q, const void* k_cache, c
     if (dtype == XR_F32)
         k_attention_ref<float><<<grid, 64, 0, stream>>>((float*)out, (const float*)q, (const float*)k_cache,
                                                         (const float*)v_cache, positions, req_of_token, block_table,
-                                                        table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window);
+                                                        table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window, slopes);
     else if (dtype == XR_BF16)
         k_attention_ref<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
                                                          (const bf16_t*)v_cache, positions, req_of_token, block_table,
-                                                         table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window);
+                                                         table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window, slopes);
     else { xr_set_error("attention: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("attention_ref");
     return XR_OK;

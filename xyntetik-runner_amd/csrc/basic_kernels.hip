@@ -149,6 +149,79 @@ extern "C" int xr_rmsnorm(void* out, const float* x, const void* w, const int* r
     return XR_OK;
 }
 
+// ---------------------------------------------------------------- dynamic tanh ("DyT")
+// A norm without statistics: y_i = tanh(alpha x_i) w_i + b_i, alpha one number, in 32-bit.  As nothing of
+// the row enters an element's value, the kernel is element-wise, and one pass can do what lies between two
+// sublayers of a layer whose sublayers are normed before and after:
+//   x += mult * (tanh(alpha_p y) w_p + b_p)        (the sublayer's result y through its second norm)
+//   h  = tanh(alpha_n x) w_n + b_n                 (the next sublayer's input)
+// either half alone too.  `rows` selects rows of x for the second half alone (the final norm).
+struct DytArgs {
+    float* x;               // [T, ldx] 32-bit residual rows
+    const void* y;          // [T, E] the sublayer's result, or null
+    const float* w_p; const float* b_p; float alpha_p, mult;
+    void* h;                // [R, E] out, or null
+    const float* w_n; const float* b_n; float alpha_n;
+    const int* rows;
+    int E, ldx;
+    size_t n;               // elements (groups of NV) in all
+};
+
+template <typename TY, typename TO, int NV>
+__global__ __launch_bounds__(256) void k_dyt_step(DytArgs a) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= a.n) return;
+    const int per_row = a.E / NV;
+    const size_t r = i / per_row;
+    const int c = (int)(i - r * per_row) * NV;
+    const size_t src = a.rows ? (size_t)a.rows[r] : r;
+    float* xp = a.x + src * a.ldx + c;
+    float v[NV];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) v[k] = xp[k];
+    if (a.y) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const float yv = ld<TY>((const TY*)a.y, r * a.E + c + k);
+            v[k] = v[k] + a.mult * fmaf(tanhf(a.alpha_p * yv), a.w_p[c + k], a.b_p[c + k]);
+            xp[k] = v[k];
+        }
+    }
+    if (a.h) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+            st<TO>((TO*)a.h, r * a.E + c + k, fmaf(tanhf(a.alpha_n * v[k]), a.w_n[c + k], a.b_n[c + k]));
+    }
+}
+
+extern "C" int xr_dyt_step(float* x, const void* y, const float* w_p, const float* b_p, float alpha_p, float mult,
+                           void* h, const float* w_n, const float* b_n, float alpha_n, const int* rows, int R, int E,
+                           int ldx, int y_dtype, int h_dtype, hipStream_t stream) {
+    XR_REQUIRE(R >= 0 && E > 0 && ldx >= E, "dyt: bad sizes R=%d E=%d ldx=%d", R, E, ldx);
+    XR_REQUIRE(x != nullptr && (y != nullptr || h != nullptr), "dyt: nothing to do");
+    XR_REQUIRE(!y || (w_p && b_p), "dyt: the norm of the sublayer's result needs its weight and bias");
+    XR_REQUIRE(!h || (w_n && b_n), "dyt: the norm needs its weight and bias");
+    XR_REQUIRE(!(y && rows), "dyt: a selection of rows goes with the norm alone");
+    XR_REQUIRE((y_dtype == XR_F32 || y_dtype == XR_BF16) && (h_dtype == XR_F32 || h_dtype == XR_BF16),
+               "dyt: bad dtypes y=%d h=%d", y_dtype, h_dtype);
+    if (R == 0) return XR_OK;
+    const bool vec = E % 4 == 0 && ldx % 4 == 0;
+    DytArgs a{x, y, w_p, b_p, alpha_p, mult, h, w_n, b_n, alpha_n, rows, E, ldx, (size_t)R * (E / (vec ? 4 : 1))};
+    const unsigned blocks = (unsigned)((a.n + 255) / 256);
+#define DY(TY, TO)                                                                  \
+    do {                                                                            \
+        if (vec) k_dyt_step<TY, TO, 4><<<blocks, 256, 0, stream>>>(a);              \
+        else k_dyt_step<TY, TO, 1><<<blocks, 256, 0, stream>>>(a);                  \
+    } while (0)
+    if (y_dtype == XR_F32 && h_dtype == XR_F32) DY(float, float);
+    else if (y_dtype == XR_F32) DY(float, bf16_t);
+    else if (h_dtype == XR_F32) DY(bf16_t, float);
+    else DY(bf16_t, bf16_t);
+#undef DY
+    XR_CHECK_LAUNCH("dyt_step");
+    return XR_OK;
+}
+
 // ---------------------------------------------------------------- rotary + cache write
 // Rotation of pair index j of a head by a = pos * inv_freq[j]:
 //   (x0, x1) -> (x0*c - x1*s, x0*s + x1*c), c = cos(a)*mscale, s = sin(a)*mscale
@@ -352,17 +425,18 @@ extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, i
 }
 
 // ---------------------------------------------------------------- residual add
+// x += scale * y (one rounding; with scale 1 the plain sum)
 template <typename TY>
-__global__ void k_add(float* __restrict__ x, const TY* __restrict__ y, size_t n) {
+__global__ void k_add(float* __restrict__ x, const TY* __restrict__ y, size_t n, float scale) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) x[i] = x[i] + ld<TY>(y, i);
+    if (i < n) x[i] = fmaf(scale, ld<TY>(y, i), x[i]);
 }
 
-extern "C" int xr_add(float* x, const void* y, size_t n, int y_dtype, hipStream_t stream) {
+extern "C" int xr_add(float* x, const void* y, size_t n, int y_dtype, float scale, hipStream_t stream) {
     if (n == 0) return XR_OK;
     unsigned blocks = (unsigned)((n + 255) / 256);
-    if (y_dtype == XR_F32) k_add<float><<<blocks, 256, 0, stream>>>(x, (const float*)y, n);
-    else if (y_dtype == XR_BF16) k_add<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)y, n);
+    if (y_dtype == XR_F32) k_add<float><<<blocks, 256, 0, stream>>>(x, (const float*)y, n, scale);
+    else if (y_dtype == XR_BF16) k_add<bf16_t><<<blocks, 256, 0, stream>>>(x, (const bf16_t*)y, n, scale);
     else { xr_set_error("add: bad dtype %d", y_dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("add");
     return XR_OK;

@@ -392,14 +392,19 @@ __global__ void k_moe_combine(float* __restrict__ y, const float* __restrict__ y
 
 // The routed experts over many rows: sort, z = relu(up)^2 by expert, yz = down by expert, y = the weighted sum.
 // scratch: ints [A + 3 * (ceil(A / 16) + n) + 1]; z: bf16 [A, F]; yz: float [A, E].
+// Gated experts (`gu` given: float [A, 2F]; w_up [n, 2F, E], an expert's gate rows before its up rows): the first
+// product leaves both branches in 32 bits and the gate's own kernel makes z = silu(gate) * up of them.
+extern "C" int xr_gate_mul(void* out, const void* gu, int T, int F, int ld_gu, int dtype, int out_dtype, int act, float param,
+                           hipStream_t stream);
 extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch, const void* h, const void* w_up,
                                       const void* w_down, const int* idx, const float* wts, int T, int E, int F, int ld_h,
-                                      int ld_y, int n, int top, int accumulate, hipStream_t stream) {
+                                      int ld_y, int n, int top, int accumulate, float* gu, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && E > 0 && F > 0 && ld_h >= E && ld_y >= E, "moe_experts_grouped: bad sizes T=%d E=%d F=%d", T, E, F);
     XR_REQUIRE(n >= 1 && n <= SORT_MAX_EXPERTS && top >= 1 && top <= n, "moe_experts_grouped: %d experts (at most %d), %d chosen", n,
                SORT_MAX_EXPERTS, top);
     XR_REQUIRE((long long)T * top <= (1 << 24), "moe_experts_grouped: too many rows");
-    XR_REQUIRE(grouped_operands_ok(h, w_up, E, ld_h, 0, (long long)F * E) && grouped_operands_ok(z, w_down, F, F, 0, (long long)E * F),
+    const int Fu = gu ? 2 * F : F;          // rows of an expert's first matrix
+    XR_REQUIRE(grouped_operands_ok(h, w_up, E, ld_h, 0, (long long)Fu * E) && grouped_operands_ok(z, w_down, F, F, 0, (long long)E * F),
                "moe_experts_grouped: widths and row strides must be multiples of 8 and the operands 16-byte aligned");
     if (T == 0) return XR_OK;
     const int A = T * top, avg = A / n;
@@ -417,9 +422,14 @@ extern "C" int xr_moe_experts_grouped(float* y, void* z, float* yz, int* scratch
     g.perm = perm; g.tile_group = tile_group; g.tile_start = tile_start; g.tile_count = tile_count; g.n_tiles = n_tiles;
     g.a_group_stride = 0; g.o_group_stride = 0;
     // up: rows of h by token, results by choice
-    g.a = (const bf16_t*)h; g.lda = ld_h; g.w = (const bf16_t*)w_up; g.w_group_stride = (long long)F * E; g.out = z; g.ldo = F;
-    g.N = F; g.K = E; g.out_bf16 = 1; g.act = GM_ACT_RELU2; g.gather_div = top;
+    g.a = (const bf16_t*)h; g.lda = ld_h; g.w = (const bf16_t*)w_up; g.w_group_stride = (long long)Fu * E;
+    g.out = gu ? (void*)gu : z; g.ldo = Fu;
+    g.N = Fu; g.K = E; g.out_bf16 = gu ? 0 : 1; g.act = gu ? GM_ACT_NONE : GM_ACT_RELU2; g.gather_div = top;
     launch_grouped(g, max_tiles, bm, stream);
+    if (gu) {
+        const int rc = xr_gate_mul(z, gu, A, F, 2 * F, XR_F32, XR_BF16, XR_ACT_SILU, 0.f, stream);
+        if (rc != XR_OK) return rc;
+    }
     // down: rows of z by choice, results by choice
     g.a = (const bf16_t*)z; g.lda = F; g.w = (const bf16_t*)w_down; g.w_group_stride = (long long)E * F; g.out = yz; g.ldo = E;
     g.N = E; g.K = F; g.out_bf16 = 0; g.act = GM_ACT_NONE; g.gather_div = 1;

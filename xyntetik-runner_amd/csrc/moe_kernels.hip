@@ -5,8 +5,11 @@
 // their weights: the chosen scores (without the correction) over their sum + 1e-20.
 // k_moe_up / k_moe_down: the experts' two products token by token, a wave an output column, the
 // weights of the chosen experts streamed: what a few decoded tokens need.  Expert:
-// down(act(up h)), act = relu squared.  The down product adds a token's experts up in the order
+// down(act(up h)), act = relu squared, or gated: down(silu(gate h) * (up h)) with the gate's rows before
+// the up rows in one matrix [2F, E].  The down product adds a token's experts up in the order
 // of its choice and writes (or adds to) 32-bit rows.
+// k_moe_table_route: the choice without a router, a row of a table [vocab, top] by the token's id, every
+// chosen expert with the same weight.
 #include "common.h"
 
 #define MOE_MAX_EXPERTS 1024
@@ -75,6 +78,27 @@ extern "C" int xr_moe_route(int* idx, float* wts, const float* logits, const flo
     return XR_OK;
 }
 
+__global__ void k_moe_table_route(int* __restrict__ idx, float* __restrict__ wts, const int* __restrict__ table,
+                                  const int* __restrict__ ids, int T, int V, int top, int n, float weight) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= T * top) return;
+    const int t = i / top, j = i - t * top;
+    int id = ids[t];
+    id = id < 0 || id >= V ? 0 : id;                    // (as the embedding reads row 0 for an id outside the vocabulary)
+    idx[i] = min(max(table[(size_t)id * top + j], 0), n - 1);
+    wts[i] = weight;
+}
+
+extern "C" int xr_moe_table_route(int* idx, float* wts, const int* table, const int* ids, int T, int V, int top, int n,
+                                  float weight, hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && V > 0 && top >= 1 && n >= 1 && top <= MOE_MAX_TOP, "moe_table_route: bad sizes T=%d V=%d top=%d n=%d", T, V, top, n);
+    XR_REQUIRE((long long)T * top <= 0x7fffffffLL, "moe_table_route: too many rows");
+    if (T == 0) return XR_OK;
+    k_moe_table_route<<<(T * top + 255) / 256, 256, 0, stream>>>(idx, wts, table, ids, T, V, top, n, weight);
+    XR_CHECK_LAUNCH("moe_table_route");
+    return XR_OK;
+}
+
 // A wave's dot product of two rows of n elements; `vec`: both rows start on 16 bytes and n is a multiple of
 // 8 (bfloat16) or 4 (float), so a lane reads 16 bytes at a time.
 template <typename TW> __device__ inline float wave_dot(const TW* __restrict__ w, const TW* __restrict__ x, int n, int lane, bool vec);
@@ -108,16 +132,25 @@ template <> __device__ inline float wave_dot<bf16_t>(const bf16_t* __restrict__ 
     return wave_sum(acc);
 }
 
-// z[t * top + j][f] = relu(W_up[e][f] . h[t])^2 for e = idx[t][j].  Grid (T * top, ceil(F / 4)); a wave a column.
+// z[t * top + j][f] = relu(W_up[e][f] . h[t])^2 for e = idx[t][j]; `gated`: silu(W_up[e][f] . h[t]) * (W_up[e][F + f] . h[t]).
+// Grid (T * top, ceil(F / 4)); a wave a column.
+#define MOE_ACT_RELU2 0
+#define MOE_ACT_SWIGLU 1
 template <typename TW>
 __global__ __launch_bounds__(256) void k_moe_up(TW* __restrict__ z, const TW* __restrict__ h, const TW* __restrict__ w_up,
-                                                const int* __restrict__ idx, int E, int F, int ld_h, int top, int n, int vec) {
+                                                const int* __restrict__ idx, int E, int F, int ld_h, int top, int n, int vec,
+                                                int gated) {
     const int a = blockIdx.x, f = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (f >= F) return;
     const int t = a / top, e = min(max(idx[a], 0), n - 1);
     const TW* row = h + (size_t)t * ld_h;
-    const TW* w = w_up + ((size_t)e * F + f) * E;
+    const TW* w = w_up + ((size_t)e * (gated ? 2 * F : F) + f) * E;
     const float acc = wave_dot<TW>(w, row, E, lane, vec != 0);
+    if (gated) {
+        const float up = wave_dot<TW>(w + (size_t)F * E, row, E, lane, vec != 0);
+        if (lane == 0) st<TW>(z, (size_t)a * F + f, gate_value<false>(XR_ACT_SILU, 0.f, acc, up));
+        return;
+    }
     if (lane == 0) {
         const float r = fmaxf(acc, 0.f);
         st<TW>(z, (size_t)a * F + f, r * r);
@@ -146,7 +179,9 @@ __global__ __launch_bounds__(256) void k_moe_down(float* __restrict__ y, const T
 
 extern "C" int xr_moe_experts(float* y, void* z, const void* h, const void* w_up, const void* w_down, const int* idx,
                               const float* wts, int T, int E, int F, int ld_h, int ld_y, int n, int top, int accumulate,
-                              int dtype, hipStream_t stream) {
+                              int dtype, int act, hipStream_t stream) {
+    XR_REQUIRE(act == MOE_ACT_RELU2 || act == MOE_ACT_SWIGLU, "moe_experts: activation %d (0 = relu squared, 1 = SiLU-gated)", act);
+    const int gated = act == MOE_ACT_SWIGLU;
     XR_REQUIRE(T >= 0 && E > 0 && F > 0 && ld_h >= E && ld_y >= E, "moe_experts: bad sizes T=%d E=%d F=%d", T, E, F);
     XR_REQUIRE(n >= 1 && top >= 1 && top <= n && top <= MOE_MAX_TOP, "moe_experts: %d experts, %d chosen", n, top);
     XR_REQUIRE((long long)T * top <= 0x7fffffffLL, "moe_experts: too many rows");
@@ -156,10 +191,10 @@ extern "C" int xr_moe_experts(float* y, void* z, const void* h, const void* w_up
     const bool al = ((uintptr_t)h % 16) == 0 && ((uintptr_t)w_up % 16) == 0 && ((uintptr_t)w_down % 16) == 0 && ((uintptr_t)z % 16) == 0;
     const int vu = al && E % per16 == 0 && ld_h % per16 == 0, vd = al && F % per16 == 0;
     if (dtype == XR_F32) {
-        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top, n, vu);
+        k_moe_up<float><<<gu, 256, 0, stream>>>((float*)z, (const float*)h, (const float*)w_up, idx, E, F, ld_h, top, n, vu, gated);
         k_moe_down<float><<<gd, 256, 0, stream>>>(y, (const float*)z, (const float*)w_down, idx, wts, E, F, ld_y, top, n, accumulate, vd);
     } else if (dtype == XR_BF16) {
-        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top, n, vu);
+        k_moe_up<bf16_t><<<gu, 256, 0, stream>>>((bf16_t*)z, (const bf16_t*)h, (const bf16_t*)w_up, idx, E, F, ld_h, top, n, vu, gated);
         k_moe_down<bf16_t><<<gd, 256, 0, stream>>>(y, (const bf16_t*)z, (const bf16_t*)w_down, idx, wts, E, F, ld_y, top, n, accumulate, vd);
     } else { xr_set_error("moe_experts: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("moe_experts");

@@ -50,7 +50,7 @@ _PROTOS = {
     "xr_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rope_kv_write": [_p, _p, _p, _i, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
     "xr_gate_mul": [_p, _p, _i, _i, _i, _i, _i, _i, _f, _p],
-    "xr_add": [_p, _p, _sz, _i, _p],
+    "xr_add": [_p, _p, _sz, _i, _f, _p],
     "xr_fill_rows": [_p, _p, _i, _sz, _u32, _p],
     "xr_fill_rows_many": [_p, _p, _i, _sz, _p, _i, _u32, _p],
     "xr_convert": [_p, _p, _sz, _i, _i, _p],
@@ -59,7 +59,11 @@ _PROTOS = {
     "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_rope_table": [_p, _p, _p, _i, _i, _f, _p],
-    "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p],
+    "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p],
+    "xr_dyt_step": [_p, _p, _p, _p, _f, _f, _p, _p, _p, _f, _p, _i, _i, _i, _i, _i, _p],
+    "xr_token_shift": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_head_rmsnorm": [_p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _f, _f, _i, _p],
+    "xr_moe_table_route": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _p],
     "xr_sample": [_p, _p, _i, _i, _i, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _p, _p],
     "xr_layernorm": [_p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
     "xr_layernorm_conv": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _p],
@@ -74,9 +78,9 @@ _PROTOS = {
     "xr_streams_step": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
     "xr_latent_prepare": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p],
     "xr_moe_route": [_p, _p, _p, _p, _i, _i, _i, _i, _p],
-    "xr_moe_experts_grouped": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_moe_experts_grouped": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p],
     "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
-    "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
+    "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
     "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
@@ -86,7 +90,9 @@ _PROTOS = {
 }
 
 CONV_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}      # XR_CONV_* of sequence_kernels.hip
-RECURRENCES = {"retention": 0, "delta": 1}              # XR_REC_* of recurrent_kernels.hip
+RECURRENCES = {"retention": 0, "delta": 1, "wkv": 2}    # XR_REC_* of recurrent_kernels.hip
+ROW_ACTIVATIONS = {"silu": 1, "tanh": 2}                # what act_rows_ applies in place
+EXPERT_ACTIVATIONS = {"relu2": 0, "swiglu": 1}          # MOE_ACT_* of moe_kernels.hip
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
@@ -263,14 +269,14 @@ class Ops:
         """``silu(gu[:, :F]) * gu[:, F:]``."""
         return self.gate_mul(gu, "silu")
 
-    def add_(self, x: torch.Tensor, y: torch.Tensor) -> None:
-        """``x += y`` with 32-bit ``x``."""
+    def add_(self, x: torch.Tensor, y: torch.Tensor, scale: float = 1.0) -> None:
+        """``x += scale * y`` with 32-bit ``x``."""
         self._dev(x, y)
         if x.dtype != torch.float32 or x.shape != y.shape:
             raise KernelError(f"add_: x must be float32 and shapes equal, got {x.dtype} {tuple(x.shape)} {tuple(y.shape)}")
         self._contig(x, "add_ x")
         self._contig(y, "add_ y")
-        self.lib.check(self.lib.xr_add(x.data_ptr(), y.data_ptr(), x.numel(), dtype_code(y.dtype), _stream()))
+        self.lib.check(self.lib.xr_add(x.data_ptr(), y.data_ptr(), x.numel(), dtype_code(y.dtype), float(scale), _stream()))
 
     def fill_rows_(self, base: torch.Tensor, rows: Optional[torch.Tensor], n_rows: int, value_bits: int = 0) -> None:
         """Set whole rows of ``base`` (first axis) to a 32-bit pattern."""
@@ -588,8 +594,9 @@ class Ops:
         return q
 
     def attention(self, q, k_cache, v_cache, ctx, group: int, H: int, Hk: int, D: int, page_size: int,
-                  scale: float, window: Optional[int] = None) -> torch.Tensor:
+                  scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Causal attention of every token of the step over its request's cached keys and values.
+        ``slopes`` (32-bit ``[H]``): ``slopes[h] * (i - j)`` is taken off the score of query i and key j.
 
         bfloat16 runs on the matrix cores (head sizes in steps of 16 up to 256, pages of at least
         16 positions); float32, and what the MFMA kernel does not take, runs the 32-bit kernel.
@@ -603,7 +610,12 @@ class Ops:
         if H % Hk:
             raise KernelError(f"attention: {H} query heads are not a multiple of {Hk} key/value heads")
         out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
-        if self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16:
+        if slopes is not None:
+            self._dev(slopes)
+            if slopes.dtype != torch.float32 or slopes.numel() != H or not slopes.is_contiguous():
+                raise KernelError(f"attention: the slopes must be float32 [{H}]")
+        if (self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16
+                and slopes is None):
             lib = self.attention_lib(D)
             plan = ctx.attention_plan(group, H // Hk, window, Hk, page_size)
             part_o = part_ml = None
@@ -619,7 +631,7 @@ class Ops:
         self.lib.check(self.lib.xr_attention_ref(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
             req_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), T, H, Hk, D, page_size,
-            float(scale), int(window or 0), dtype_code(q.dtype), _stream()))
+            float(scale), int(window or 0), dtype_code(q.dtype), _ptr(slopes), _stream()))
         return out
 
     def attention_lib(self, D: int) -> "_Lib":
@@ -649,6 +661,84 @@ class Ops:
         self.lib.check(self.lib.xr_layernorm(out.data_ptr(), x.data_ptr(), _ptr(w), _ptr(rows), R, E, x.stride(0),
                                              float(eps), dtype_code(out_dtype), _stream()))
         return out
+
+    def dyt(self, x: torch.Tensor, alpha: float, w: torch.Tensor, b: torch.Tensor, out_dtype: torch.dtype,
+            rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Dynamic tanh of the rows of 32-bit ``x`` (or of the rows ``rows`` selects): ``tanh(alpha x) * w + b``,
+        a norm that takes no statistic of the row; ``w`` and ``b`` 32-bit ``[E]``."""
+        return self.dyt_step(x, norm=(alpha, w, b), out_dtype=out_dtype, rows=rows)
+
+    def dyt_step(self, x: torch.Tensor, y: Optional[torch.Tensor] = None, post=None, mult: float = 1.0, norm=None,
+                 out_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+        """What lies between two sublayers that are normed before and after, in one pass over the 32-bit
+        residual rows ``x [T, E]``: with ``y [T, E]`` (a sublayer's result, 32-bit or the compute dtype) and
+        ``post`` = (alpha, w, b): ``x += mult * (tanh(alpha y) w + b)`` in place; with ``norm`` = (alpha, w, b):
+        ``tanh(alpha x) w + b`` of the rows (updated or not) comes back in ``out_dtype``.  Either half alone too."""
+        self._dev(x, y, rows)
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
+            raise KernelError("dyt: x must be float32 [rows, width] with unit column stride")
+        E = x.shape[1]
+        for part in (post, norm):
+            if part is not None:
+                _, w, b = part
+                self._dev(w, b)
+                if any(t.dtype != torch.float32 or t.numel() != E or not t.is_contiguous() for t in (w, b)):
+                    raise KernelError(f"dyt: weight and bias must be float32 [{E}]")
+        if (y is None) != (post is None):
+            raise KernelError("dyt: a sublayer's result and its norm come together")
+        if y is not None and (tuple(y.shape) != tuple(x.shape) or not y.is_contiguous() or rows is not None):
+            raise KernelError(f"dyt: y must be contiguous {tuple(x.shape)} and the rows all")
+        R = x.shape[0] if rows is None else rows.numel()
+        h = torch.empty((R, E), dtype=out_dtype or torch.float32, device=x.device) if norm is not None else None
+        self.lib.check(self.lib.xr_dyt_step(
+            x.data_ptr(), _ptr(y), _ptr(post[1]) if post else None, _ptr(post[2]) if post else None,
+            float(post[0]) if post else 0.0, float(mult), _ptr(h), _ptr(norm[1]) if norm else None,
+            _ptr(norm[2]) if norm else None, float(norm[0]) if norm else 0.0, _ptr(rows), R, E, x.stride(0),
+            dtype_code(y.dtype) if y is not None else XR_F32, dtype_code(h.dtype) if h is not None else XR_F32, _stream()))
+        return h
+
+    def token_shift(self, h: torch.Tensor, mu: torch.Tensor, state: torch.Tensor, ctx, out_dtype: torch.dtype) -> torch.Tensor:
+        """``out[t, s] = h[t] + (h[t - 1] - h[t]) * mu[s]`` for the ``n`` mixes ``mu [n, E]`` (32-bit) of the 32-bit rows
+        ``h [T, E]``, as ``[T, n * E]`` in ``out_dtype``.  The row before a request's first row of the step is its row
+        of ``state [slots + 1, E]`` (zero for a request that begins), which is brought up to date."""
+        self._dev(h, mu, state)
+        if h.dtype != torch.float32 or h.dim() != 2 or h.stride(1) != 1:
+            raise KernelError("token_shift: h must be float32 [rows, width] with unit column stride")
+        T, E = h.shape
+        if mu.dtype != torch.float32 or mu.dim() != 2 or mu.shape[1] != E or not mu.is_contiguous():
+            raise KernelError(f"token_shift: the mixes must be float32 [n, {E}]")
+        if state.dtype != torch.float32 or tuple(state.shape[1:]) != (E,) or not state.is_contiguous():
+            raise KernelError(f"token_shift: state must be float32 [slots, {E}]")
+        n = mu.shape[0]
+        out = torch.empty((T, n * E), dtype=out_dtype, device=h.device)
+        self.lib.check(self.lib.xr_token_shift(out.data_ptr(), h.data_ptr(), mu.data_ptr(), state.data_ptr(), ctx.cu_q.data_ptr(),
+                                               ctx.slots.data_ptr(), ctx.req_of_token.data_ptr(), T, ctx.B, E, n, h.stride(0),
+                                               dtype_code(out_dtype), 1 if (ctx.max_q_len == 1 and T == ctx.B) else 0, _stream()))
+        return out
+
+    def head_rmsnorm_(self, q: Optional[torch.Tensor], k: Optional[torch.Tensor], wq: Optional[torch.Tensor],
+                      wk: Optional[torch.Tensor], eps: float, positions: Optional[torch.Tensor] = None,
+                      temp_coef: float = 0.0, temp_every: int = 0) -> None:
+        """In place on the 32-bit views ``q [T, H, D]`` and ``k [T, Hk, D]`` (one row stride): every head over its
+        root mean square times a weight ``[D]`` that the heads share (``wq`` / ``wk``; absent: that side stays);
+        with ``temp_every`` > 0 the queries at position p also times ``1 + temp_coef ln(floor((p + 1) / temp_every) + 1)``."""
+        self._dev(q, k, wq, wk, positions)
+        views = [t for t in (q, k) if t is not None]
+        if not views:
+            return
+        if any(t.dtype != torch.float32 or t.dim() != 3 or t.stride(2) != 1 or t.stride(1) != t.shape[2] for t in views):
+            raise KernelError("head_rmsnorm_: q and k must be float32 views [rows, heads, size] with the heads side by side")
+        one_row = views[0].shape[0] <= 1        # (a single row has no stride to speak of)
+        if (not one_row and len({t.stride(0) for t in views}) != 1) or len({t.shape[2] for t in views}) != 1:
+            raise KernelError("head_rmsnorm_: q and k must share a row stride and a head size")
+        D = views[0].shape[2]
+        for w in (wq, wk):
+            if w is not None and (w.dtype != torch.float32 or w.numel() != D or not w.is_contiguous()):
+                raise KernelError(f"head_rmsnorm_: a weight must be float32 [{D}]")
+        self.lib.check(self.lib.xr_head_rmsnorm(_ptr(q), _ptr(k), views[0].stride(0), _ptr(wq), _ptr(wk), _ptr(positions),
+                                                views[0].shape[0], q.shape[1] if q is not None else 0,
+                                                k.shape[1] if k is not None else 0, D, float(eps), float(temp_coef),
+                                                int(temp_every), _stream()))
 
     def causal_conv(self, u: torch.Tensor, w: torch.Tensor, state: Optional[torch.Tensor], ctx, out_dtype: torch.dtype,
                     residual: bool = False, activation: Optional[str] = None) -> torch.Tensor:
@@ -755,9 +845,9 @@ class Ops:
         self._dev(x)
         if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
             raise KernelError("act_rows_: x must be a float32 view [rows, width] with unit column stride")
-        if activation != "silu":
-            raise KernelError(f"act_rows_: activation {activation!r} is not built (silu)")
-        self.lib.check(self.lib.xr_act_rows(x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), CONV_ACTIVATIONS[activation], _stream()))
+        if activation not in ROW_ACTIVATIONS:
+            raise KernelError(f"act_rows_: activation {activation!r} is not built ({', '.join(sorted(ROW_ACTIVATIONS))})")
+        self.lib.check(self.lib.xr_act_rows(x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), ROW_ACTIVATIONS[activation], _stream()))
 
     # -- an embedding with a hashed table of token pairs --------------------------
     def embedding_pairs(self, table: torch.Tensor, pairs: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], ids, ctx,
@@ -921,22 +1011,42 @@ class Ops:
                                              logits.stride(0), n, int(top), _stream()))
         return idx, wts
 
+    def table_route(self, table: torch.Tensor, ids: torch.Tensor, n_experts: int):
+        """``(experts [T, top] int32, weights [T, top] float32)`` without a router: row ``ids[t]`` of ``table
+        [vocab, top]`` (int32), every chosen expert with the weight ``1 / top``."""
+        self._dev(table, ids)
+        if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
+            raise KernelError("table_route: the table must be contiguous int32 [vocab, top]")
+        V, top = table.shape
+        T = ids.numel()
+        idx = torch.empty((T, top), dtype=torch.int32, device=table.device)
+        wts = torch.empty((T, top), dtype=torch.float32, device=table.device)
+        self.lib.check(self.lib.xr_moe_table_route(idx.data_ptr(), wts.data_ptr(), table.data_ptr(), ids.data_ptr(), T, V, top,
+                                                   int(n_experts), 1.0 / top, _stream()))
+        return idx, wts
+
     GROUPED_EXPERTS_FROM = 32       # choices (rows x top) from which the experts' rows are sorted and run on the matrix cores
 
     def moe_experts(self, h: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor,
-                    out: Optional[torch.Tensor] = None, accumulate: bool = False) -> torch.Tensor:
+                    out: Optional[torch.Tensor] = None, accumulate: bool = False, activation: str = "relu2") -> torch.Tensor:
         """``out[t] (+)= sum_j wts[t, j] * w_down[e] @ relu(w_up[e] @ h[t])^2`` with ``e = idx[t, j]``, as 32-bit
-        rows; ``w_up [n, F, E]`` and ``w_down [n, E, F]`` in ``h``'s dtype.  A few choices stream the chosen
+        rows; ``w_up [n, F, E]`` and ``w_down [n, E, F]`` in ``h``'s dtype.  ``activation`` "swiglu": gated experts,
+        ``w_down[e] @ (silu(g) * u)`` with ``[g; u] = w_up[e] @ h[t]`` for ``w_up [n, 2F, E]`` (an expert's gate rows
+        before its up rows).  A few choices stream the chosen
         experts' weights, a wave an output column; from ``GROUPED_EXPERTS_FROM`` choices on (bfloat16, widths
         that are multiples of 8) the rows are sorted by expert on the device, both products run on the matrix
         cores and a last kernel adds a token's experts up in the order of its choice."""
         self._dev(h, w_up, w_down, idx, wts, out)
         T, E = h.shape
-        n, F, _ = w_up.shape
+        if activation not in EXPERT_ACTIVATIONS:
+            raise KernelError(f"moe_experts: activation {activation!r} (known: {sorted(EXPERT_ACTIVATIONS)})")
+        gated = activation == "swiglu"
+        n, Fu, _ = w_up.shape
+        F = Fu // 2 if gated else Fu
         top = idx.shape[1]
         if h.stride(1) != 1 or w_up.dtype != h.dtype or w_down.dtype != h.dtype:
             raise KernelError("moe_experts: h must have unit column stride and the experts its dtype")
-        if tuple(w_up.shape) != (n, F, E) or tuple(w_down.shape) != (n, E, F) or not w_up.is_contiguous() or not w_down.is_contiguous():
+        if tuple(w_up.shape) != (n, 2 * F if gated else F, E) or tuple(w_down.shape) != (n, E, F) or not w_up.is_contiguous() or not w_down.is_contiguous():
             raise KernelError("moe_experts: the experts' weights must be contiguous [n, F, E] and [n, E, F]")
         if idx.dtype != torch.int32 or wts.dtype != torch.float32 or tuple(idx.shape) != (T, top) or tuple(wts.shape) != (T, top):
             raise KernelError("moe_experts: the choice must be int32 [T, top] with float32 weights")
@@ -953,14 +1063,16 @@ class Ops:
             A = T * top
             yz = torch.empty((A, E), dtype=torch.float32, device=h.device)
             scratch = torch.empty((A + 3 * (-(-A // 16) + n) + 1,), dtype=torch.int32, device=h.device)
+            gu = torch.empty((A, 2 * F), dtype=torch.float32, device=h.device) if gated else None
             self.lib.check(self.lib.xr_moe_experts_grouped(out.data_ptr(), z.data_ptr(), yz.data_ptr(), scratch.data_ptr(),
                                                            h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(), idx.data_ptr(),
                                                            wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
-                                                           1 if accumulate else 0, _stream()))
+                                                           1 if accumulate else 0, _ptr(gu), _stream()))
             return out
         self.lib.check(self.lib.xr_moe_experts(out.data_ptr(), z.data_ptr(), h.data_ptr(), w_up.data_ptr(), w_down.data_ptr(),
                                                idx.data_ptr(), wts.data_ptr(), T, E, F, h.stride(0), out.stride(0), n, top,
-                                               1 if accumulate else 0, dtype_code(h.dtype), _stream()))
+                                               1 if accumulate else 0, dtype_code(h.dtype), EXPERT_ACTIVATIONS[activation],
+                                               _stream()))
         return out
 
     def delta_prepare_(self, q, k, b, a, a_log, dt_bias, G: int, H: int, D: int, q_scale: float, unit_eps: float) -> None:
@@ -993,7 +1105,9 @@ class Ops:
         """The read-outs ``[T, H * Dv]`` (32-bit) of a linear recurrence over every request's rows,
         from and into ``state [slots + 1, *recurrence_state_shape]``.  ``kind`` "retention":
         ``S <- decay_h S + k v^T`` with ``decay [H]``; "delta": ``S <- g S; u = beta (v - S^T k);
-        S <- S + k u^T`` with ``beta``/``gate [T, H]``; ``o = S^T q`` after the update in both.
+        S <- S + k u^T`` with ``beta``/``gate [T, H]``; ``o = S^T q`` after the update in both.  "wkv":
+        ``o = (S + diag(u) k v^T)^T q`` before the update ``S <- diag(w) S + k v^T``, with ``w = exp(-exp(x))``
+        a token, head and key channel from ``gate`` = x ``[T, H * D]`` and the bonus ``decay`` = u ``[H, D]``.
         ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride.  ``activation`` "silu":
         q, k and v pass SiLU on their way into the kernel (the views themselves stay as they are)."""
         if activation not in (None, "silu"):
@@ -1017,6 +1131,10 @@ class Ops:
         if kind == "delta":
             if beta is None or gate is None or tuple(beta.shape) != (T, H) or tuple(gate.shape) != (T, H):
                 raise KernelError("linear_recurrence: the delta rule needs beta and gate [T, H]")
+        elif kind == "wkv":
+            if (G != H or beta is not None or activation is not None or gate is None or tuple(gate.shape) != (T, H * D)
+                    or decay is None or decay.dtype != torch.float32 or decay.numel() != H * D or not decay.is_contiguous()):
+                raise KernelError(f"linear_recurrence: wkv needs a key head a head, decays [T, {H * D}] and float32 bonus [{H}, {D}]")
         elif decay is None or decay.dtype != torch.float32 or decay.numel() != H:
             raise KernelError(f"linear_recurrence: retention needs float32 decay [{H}]")
         out = torch.empty((T, H * Dv), dtype=torch.float32, device=q.device)

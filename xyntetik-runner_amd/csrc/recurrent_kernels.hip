@@ -2,6 +2,9 @@
 //
 //   retention:   S <- decay_h S + k v^T;                            o = S^T q
 //   delta rule:  S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   wkv:         o = (S + diag(u) k v^T)^T r;  S <- diag(w) S + k v^T    (the read-out comes before the update and
+//                gives the token itself a weight u of its own; w = exp(-exp(x)) is a decay a token, head and key
+//                channel, made here from x as the rows are fetched)
 //
 // S is [D, Dv] and its columns never meet: column c only needs v[c].  A group of R adjacent lanes
 // owns one column (lane r the rows r, r+R, r+2R, ...), keeps it in registers over the whole
@@ -20,6 +23,7 @@
 #define REC_TOKENS 16        // tokens staged at a time
 #define XR_REC_RETENTION 0
 #define XR_REC_DELTA 1
+#define XR_REC_WKV 2
 
 static inline int rec_lanes(int D) { return D > 32 ? 16 : 4; }
 
@@ -29,8 +33,8 @@ struct RecArgs {
     const float* k;
     const float* v;          // H heads of Dv
     const float* beta;       // [T, ld_g] at head 0 (delta rule)
-    const float* gate;       // [T, ld_g] at head 0: the decay of every token and head (delta rule)
-    const float* decay;      // [H] (retention)
+    const float* gate;       // [T, ld_g] at head 0: the decay of every token and head (delta rule); wkv: x of the decay, H heads of D
+    const float* decay;      // [H] (retention); wkv: the bonus u [H, D]
     float* state;
     const int* cu_q;
     const int* slots;
@@ -68,6 +72,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
     constexpr int COLS = 256 / R;
     __shared__ float4 qs[REC_TOKENS][R * DPER / 4];        // [token][r * (DPER/4) + j/4] as lanes read them
     __shared__ float4 ks[REC_TOKENS][R * DPER / 4];
+    __shared__ float4 ws[MODE == XR_REC_WKV ? REC_TOKENS : 1][R * DPER / 4];      // (wkv) the decays, as the keys lie
     __shared__ float vs[REC_TOKENS][COLS];
     __shared__ float bs[REC_TOKENS], gs[REC_TOKENS];
     const int h = blockIdx.y, tid = threadIdx.x;
@@ -95,12 +100,16 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
     const float dec = MODE == XR_REC_RETENTION ? a.decay[h] : 1.f;
     float* qf = reinterpret_cast<float*>(&qs[0][0]);
     float* kf = reinterpret_cast<float*>(&ks[0][0]);
+    float* wf = reinterpret_cast<float*>(&ws[0][0]);
+    float ub[DPER];                 // (wkv) the bonus of this lane's rows
+#pragma unroll
+    for (int j = 0; j < DPER; ++j) ub[j] = (MODE == XR_REC_WKV && R * j + r < a.D) ? a.decay[(size_t)h * a.D + R * j + r] : 0.f;
 
     // A chunk's queries, keys, values and gates go from memory into registers while the chunk before
     // it is computed, and from there into LDS: the chain of tokens never waits for memory.
     constexpr int NQ = REC_TOKENS * R * DPER / 256;       // staged elements of q (and of k) a lane
     constexpr int NV = (REC_TOKENS * COLS + 255) / 256;
-    float rq[NQ], rk[NQ], rv[NV], rb = 0.f, rg = 0.f;
+    float rq[NQ], rk[NQ], rw[MODE == XR_REC_WKV ? NQ : 1], rv[NV], rb = 0.f, rg = 0.f;
     auto fetch = [&](int c0) {
         const int nt = n - c0 < REC_TOKENS ? n - c0 : REC_TOKENS;
 #pragma unroll
@@ -113,6 +122,8 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
             rq[i] = ok ? a.q[row] : 0.f;
             rk[i] = ok ? a.k[row] : 0.f;
             if (a.act) { rq[i] = rq[i] / (1.0f + expf(-rq[i])); rk[i] = rk[i] / (1.0f + expf(-rk[i])); }
+            if (MODE == XR_REC_WKV)
+                rw[i] = ok ? expf(-expf(a.gate[(size_t)(row0 + c0 + tt) * a.ld_g + (size_t)h * a.D + d])) : 0.f;
         }
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
@@ -138,7 +149,10 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
         __syncthreads();
         // element d = R j + rr of a token goes to place rr * DPER + j; places past D hold zero
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) { qf[tid + i * 256] = rq[i]; kf[tid + i * 256] = rk[i]; }
+        for (int i = 0; i < NQ; ++i) {
+            qf[tid + i * 256] = rq[i]; kf[tid + i * 256] = rk[i];
+            if (MODE == XR_REC_WKV) wf[tid + i * 256] = rw[i];
+        }
 #pragma unroll
         for (int i = 0; i < NV; ++i)
             if (tid + i * 256 < REC_TOKENS * COLS) (&vs[0][0])[tid + i * 256] = rv[i];
@@ -173,6 +187,42 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
                     qp[j >> 2] = qq[j >> 2];
                 }
                 prev_row = row0 + c0 + tt;
+            }
+        } else if (MODE == XR_REC_WKV) {
+            // The chain is one multiply-add a token, as retention's; the read-out is of the state before the
+            // update plus the token's own k v^T times the bonus.  Four tokens' read-outs run side by side.
+            auto token = [&](int tt) {
+                const float4* kq = &ks[tt][r * (DPER / 4)];
+                const float4* qq = &qs[tt][r * (DPER / 4)];
+                const float4* wq = &ws[tt][r * (DPER / 4)];
+                const float vv = vs[tt][cl];
+                float o0 = 0.f, o1 = 0.f;
+#pragma unroll
+                for (int j = 0; j < DPER; j += 4) {
+                    const float4 kk = kq[j >> 2], q4 = qq[j >> 2], w4 = wq[j >> 2];
+                    const float t0 = kk.x * vv, t1 = kk.y * vv, t2 = kk.z * vv, t3 = kk.w * vv;
+                    o0 = fmaf(q4.x, fmaf(ub[j], t0, S[j]), o0); o1 = fmaf(q4.y, fmaf(ub[j + 1], t1, S[j + 1]), o1);
+                    o0 = fmaf(q4.z, fmaf(ub[j + 2], t2, S[j + 2]), o0); o1 = fmaf(q4.w, fmaf(ub[j + 3], t3, S[j + 3]), o1);
+                    S[j] = fmaf(w4.x, S[j], t0); S[j + 1] = fmaf(w4.y, S[j + 1], t1);
+                    S[j + 2] = fmaf(w4.z, S[j + 2], t2); S[j + 3] = fmaf(w4.w, S[j + 3], t3);
+                }
+                return o0 + o1;
+            };
+            int tt = 0;
+            for (; tt + 4 <= nt; tt += 4) {
+                float oo[4];
+#pragma unroll
+                for (int x = 0; x < 4; ++x) oo[x] = token(tt + x);
+#pragma unroll
+                for (int x = 0; x < 4; ++x) oo[x] = group_sum<R>(oo[x]);
+                if (live && r == 0) {
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) a.out[((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col] = oo[x];
+                }
+            }
+            for (; tt < nt; ++tt) {
+                const float o = group_sum<R>(token(tt));
+                if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
             }
         } else {
             // Retention's chain is one multiply-add a token; four tokens' read-outs run side by side.
@@ -280,9 +330,11 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
                                     int chunk_len, int n_chunks, float* scratch, int act, hipStream_t stream) {
     XR_REQUIRE(B >= 0 && H > 0 && G > 0 && H % G == 0, "recurrence: %d heads over %d key heads", H, G);
     XR_REQUIRE(D > 0 && D <= 256 && Dv > 0, "recurrence: key size %d (1 to 256), value size %d", D, Dv);
-    XR_REQUIRE(mode == XR_REC_RETENTION || mode == XR_REC_DELTA, "recurrence: mode %d", mode);
-    XR_REQUIRE(mode == XR_REC_RETENTION ? decay != nullptr : (beta != nullptr && gate != nullptr),
+    XR_REQUIRE(mode == XR_REC_RETENTION || mode == XR_REC_DELTA || mode == XR_REC_WKV, "recurrence: mode %d", mode);
+    XR_REQUIRE(mode == XR_REC_RETENTION ? decay != nullptr : mode == XR_REC_DELTA ? (beta != nullptr && gate != nullptr)
+                                                                                   : (gate != nullptr && decay != nullptr),
                "recurrence: the mode's gates are missing");
+    XR_REQUIRE(mode != XR_REC_WKV || (G == H && ld_g >= H * D && act == 0), "recurrence: wkv has a key head a head and decays of %d x %d a row", H, D);
     XR_REQUIRE(out && q && k && v && state && cu_q && slots, "recurrence: a pointer is missing");
     XR_REQUIRE(act == 0 || act == 1, "recurrence: activation %d of q, k and v (0: none, 1: SiLU)", act);
     if (B == 0) return XR_OK;
@@ -301,6 +353,7 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
         else k_recurrence<M, 16, 16><<<grid, 256, 0, stream>>>(a);                      \
     } while (0)
     if (mode == XR_REC_DELTA) REC(XR_REC_DELTA);
+    else if (mode == XR_REC_WKV) REC(XR_REC_WKV);
     else REC(XR_REC_RETENTION);
     if (chunks) {
         const int per_head = per * Dv * R;

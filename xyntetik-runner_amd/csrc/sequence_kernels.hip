@@ -203,6 +203,56 @@ extern "C" int xr_causal_conv(void* out, const void* u, const float* w, void* st
     return XR_OK;
 }
 
+// ---------------------------------------------------------------- mixes of a row with the row before it
+// out[t][s][c] = h[t][c] + (h[t-1][c] - h[t][c]) * mu[s][c] for n mixes s ("token shift"); the row before a
+// portion's first row is the request's state row (zero for a request that begins), which afterwards holds
+// the portion's last row.  As for the convolution above, a second kernel rewrites the state once every row
+// has been read, and in a step of one row a request (`fuse`) the row's own thread does.
+template <typename TO>
+__global__ __launch_bounds__(256) void k_token_shift(TO* __restrict__ out, const float* __restrict__ h,
+                                                     const float* __restrict__ mu, float* state,
+                                                     const int* __restrict__ cu_q, const int* __restrict__ slots,
+                                                     const int* __restrict__ req_of_token, int E, int n, int ld_h, int fuse) {
+    const int t = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= E) return;
+    const int b = req_of_token[t];
+    const bool first = t == cu_q[b];
+    float* srow = state + (size_t)slots[b] * E;
+    const float cur = h[(size_t)t * ld_h + c];
+    const float before = first ? srow[c] : h[(size_t)(t - 1) * ld_h + c];
+    const float d = before - cur;
+    for (int s = 0; s < n; ++s) st<TO>(out, ((size_t)t * n + s) * E + c, fmaf(d, mu[(size_t)s * E + c], cur));
+    if (fuse) srow[c] = cur;
+}
+
+__global__ __launch_bounds__(256) void k_shift_state(float* __restrict__ state, const float* __restrict__ h,
+                                                     const int* __restrict__ cu_q, const int* __restrict__ slots, int E, int ld_h) {
+    const int b = blockIdx.y;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= E) return;
+    const int end = cu_q[b + 1];
+    if (end <= cu_q[b]) return;
+    state[(size_t)slots[b] * E + c] = h[(size_t)(end - 1) * ld_h + c];
+}
+
+extern "C" int xr_token_shift(void* out, const float* h, const float* mu, float* state, const int* cu_q, const int* slots,
+                              const int* req_of_token, int T, int B, int E, int n, int ld_h, int out_dtype, int one_row_each,
+                              hipStream_t stream) {
+    XR_REQUIRE(T >= 0 && B >= 0 && E > 0 && n > 0 && ld_h >= E, "token_shift: bad sizes T=%d B=%d E=%d n=%d ld=%d", T, B, E, n, ld_h);
+    XR_REQUIRE(out && h && mu && state && cu_q && slots && req_of_token, "token_shift: a pointer is missing");
+    XR_REQUIRE(!one_row_each || T == B, "token_shift: %d rows of %d requests are not one row each", T, B);
+    XR_REQUIRE(out_dtype == XR_F32 || out_dtype == XR_BF16, "token_shift: bad dtype %d", out_dtype);
+    if (T == 0 || B == 0) return XR_OK;
+    const int fuse = one_row_each ? 1 : 0;
+    const dim3 grid((E + 255) / 256, T), sgrid((E + 255) / 256, B);
+    if (out_dtype == XR_F32) k_token_shift<float><<<grid, 256, 0, stream>>>((float*)out, h, mu, state, cu_q, slots, req_of_token, E, n, ld_h, fuse);
+    else k_token_shift<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, h, mu, state, cu_q, slots, req_of_token, E, n, ld_h, fuse);
+    if (!fuse) k_shift_state<<<sgrid, 256, 0, stream>>>(state, h, cu_q, slots, E, ld_h);
+    XR_CHECK_LAUNCH("token_shift");
+    return XR_OK;
+}
+
 // Layer norm and the convolution behind it in one kernel, for a step in which every request
 // brings one row: row b is request b's, its convolution reads the request's carried inputs and
 // the row itself, and the thread that owns a channel moves that channel's carried inputs on.
@@ -402,19 +452,20 @@ extern "C" int xr_gated_rmsnorm(void* out, const float* o, const float* gate, co
 }
 
 // ---------------------------------------------------------------- an activation on 32-bit rows, in place
-// x[t][c] <- act(x[t][c]) for the first W columns of rows of stride ld; act 1 = SiLU.
+// x[t][c] <- act(x[t][c]) for the first W columns of rows of stride ld; act 1 = SiLU, 2 = tanh.
+#define XR_ACT_ROWS_TANH 2
 __global__ void k_act_rows(float* __restrict__ x, int W, int ld, size_t n, int act) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t t = i / W;
     float* p = x + t * ld + (i - t * W);
     const float v = *p;
-    *p = v / (1.0f + expf(-v));
+    *p = act == XR_ACT_ROWS_TANH ? tanhf(v) : v / (1.0f + expf(-v));
 }
 
 extern "C" int xr_act_rows(float* x, int T, int W, int ld, int act, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && W > 0 && ld >= W, "act_rows: bad sizes T=%d W=%d ld=%d", T, W, ld);
-    XR_REQUIRE(act == XR_CONV_SILU, "act_rows: activation %d is not built (1 = SiLU)", act);
+    XR_REQUIRE(act == XR_CONV_SILU || act == XR_ACT_ROWS_TANH, "act_rows: activation %d is not built (1 = SiLU, 2 = tanh)", act);
     const size_t n = (size_t)T * W;
     if (n == 0) return XR_OK;
     k_act_rows<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, W, ld, n, act);

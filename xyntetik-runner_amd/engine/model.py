@@ -28,7 +28,9 @@ class Model:
                 make_part("feed_forward", ls.feed_forward) if ls.feed_forward is not None else None,
                 {name: make_part("norm", ps) for name, ps in ls.norms.items()},
                 {name: make_part("filter", ps) for name, ps in ls.filters.items()},
-                {name: make_part("connection", ps) for name, ps in ls.connections.items()}))
+                {name: make_part("connection", ps) for name, ps in ls.connections.items()},
+                ls.block_params))
+        self.injection = make_part("injection", spec.injection) if spec.injection is not None else None
         self.final_norm = make_part("norm", spec.final_norm)
         self.head = make_part("head", spec.head)
         self.rt: Optional[Runtime] = None
@@ -38,6 +40,8 @@ class Model:
     # ------------------------------------------------------------------ tensors
     def _named_parts(self):
         yield self.spec.embedding.prefix, self.embedding
+        if self.injection is not None:
+            yield self.spec.injection.prefix, self.injection
         for ls, blk in zip(self.spec.layers, self.blocks):
             for name, ps in ls.norms.items():
                 yield ps.prefix, blk.norms[name]
@@ -120,11 +124,15 @@ class Model:
         if self.spec.streams is not None:       # the layers keep several copies of the residual stream
             x = ctx.ops.streams_expand(x, self.spec.streams)
         order = self.spec.order
+        x0 = self.injection.prepare(ctx, x) if self.injection is not None else None
         h = None            # the result of the next block's first norm, if the block before made it
         for i, step in enumerate(order):
             block = self.blocks[step.layer]
+            if step.enters:         # (the block before made no input for this one: the stream it would have read is remade here)
+                x = self.injection.forward(ctx, x, x0)
             if block.chained:
-                after = self.blocks[order[i + 1].layer].entry_norm() if i + 1 < len(order) else None
+                chain = i + 1 < len(order) and not order[i + 1].enters
+                after = self.blocks[order[i + 1].layer].entry_norm() if chain else None
                 h = block.forward(ctx, caches[i], x, h=h, after=after)
             else:
                 block.forward(ctx, caches[i], x)

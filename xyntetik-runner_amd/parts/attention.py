@@ -10,6 +10,12 @@ encoding rotates q and k; k and v go to the cache (k rotated, v as it is); query
 The three input projections are kept as one ``[Q + 2K, E]`` matrix.  A layer that
 reads another layer's cache (``kv_shared``) has no key or value projection and writes
 nothing (src/model.h:492-494).
+
+Options that other designs bring: ``values="keys"``: there is no value projection and the values are the
+keys as projected (before any transform of queries and keys: the cache then holds the transformed keys
+and, as values, the untransformed ones); ``slopes``: one number a query head, ``slopes[h] * (i - j)`` is
+taken off the score of query i and key j, a bias that grows with the distance and stands in for a position
+encoding; ``weight_suffix`` / ``bias_suffix``: how a checkpoint names a projection's matrix and bias.
 """
 from __future__ import annotations
 
@@ -30,7 +36,8 @@ class PagedAttention(Mixer):
                  position=None, window: Optional[int] = None, scale: Optional[float] = None,
                  bias: bool = False, out_bias: Optional[bool] = None, kv_shared: bool = False, qk_transform=None,
                  q_name: str = "q_proj", k_name: str = "k_proj", v_name: str = "v_proj",
-                 o_name: str = "o_proj"):
+                 o_name: str = "o_proj", values: str = "projection", slopes=None, weight_suffix: str = ".weight",
+                 bias_suffix: str = ".bias"):
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads are not a multiple of {num_kv_heads} key/value heads")
         if window is not None and window < 1:
@@ -45,6 +52,14 @@ class PagedAttention(Mixer):
         self.bias = bool(bias)
         self.out_bias = self.bias if out_bias is None else bool(out_bias)
         self.kv_shared = bool(kv_shared)
+        if values not in ("projection", "keys"):
+            raise ValueError(f"attention: values come from their 'projection' or are the 'keys', not {values!r}")
+        self.values_are_keys = values == "keys"
+        if slopes is not None and len(slopes) != int(num_heads):
+            raise ValueError(f"attention: {len(slopes)} slopes for {num_heads} query heads")
+        self.slope_values = [float(s) for s in slopes] if slopes is not None else None
+        self.w_sfx, self.b_sfx = weight_suffix, bias_suffix
+        self.slopes = None
         self.names = (q_name, k_name, v_name, o_name)
         self.position = make_part("position", position) if position is not None else None
         # applied to the 32-bit projections before the position encoding; with one, the projections
@@ -61,17 +76,20 @@ class PagedAttention(Mixer):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E, Q, K = self.hidden_size, self.q_size, self.kv_size
         q, k, v, o = self.names
-        specs = {f"{q}.weight": ParamSpec((Q, E)), f"{o}.weight": ParamSpec((E, Q))}
+        ws, bs = self.w_sfx, self.b_sfx
+        specs = {f"{q}{ws}": ParamSpec((Q, E)), f"{o}{ws}": ParamSpec((E, Q))}
         if not self.kv_shared:
-            specs[f"{k}.weight"] = ParamSpec((K, E))
-            specs[f"{v}.weight"] = ParamSpec((K, E))
+            specs[f"{k}{ws}"] = ParamSpec((K, E))
+            if not self.values_are_keys:
+                specs[f"{v}{ws}"] = ParamSpec((K, E))
         if self.bias:
-            specs[f"{q}.bias"] = ParamSpec((Q,), role="vector", init="normal")
+            specs[f"{q}{bs}"] = ParamSpec((Q,), role="vector", init="normal")
             if not self.kv_shared:
-                specs[f"{k}.bias"] = ParamSpec((K,), role="vector", init="normal")
-                specs[f"{v}.bias"] = ParamSpec((K,), role="vector", init="normal")
+                specs[f"{k}{bs}"] = ParamSpec((K,), role="vector", init="normal")
+                if not self.values_are_keys:
+                    specs[f"{v}{bs}"] = ParamSpec((K,), role="vector", init="normal")
         if self.out_bias:
-            specs[f"{o}.bias"] = ParamSpec((E,), role="vector", init="normal")
+            specs[f"{o}{bs}"] = ParamSpec((E,), role="vector", init="normal")
         if self.qk_transform is not None:
             for name, ps in self.qk_transform.param_specs().items():
                 if name in specs:
@@ -92,16 +110,21 @@ class PagedAttention(Mixer):
             self.qk_transform.bind({n: tensors[n] for n in self.qk_transform.param_specs()}, rt)
         q, k, v, o = self.names
         H, Hk, D = self.num_heads, self.num_kv_heads, self.head_dim
-        mats = [tensors[f"{q}.weight"]]
+        ws, bsf = self.w_sfx, self.b_sfx
+        if self.values_are_keys:        # the value projection is the key projection: its rows stand twice in the one matrix
+            v = k
+        mats = [tensors[f"{q}{ws}"]]
         if not self.kv_shared:
-            mats += [tensors[f"{k}.weight"], tensors[f"{v}.weight"]]
+            mats += [tensors[f"{k}{ws}"], tensors[f"{v}{ws}"]]
         w_in = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
         b_in = None
         if self.bias:
-            bs = [tensors[f"{q}.bias"]]
+            bs = [tensors[f"{q}{bsf}"]]
             if not self.kv_shared:
-                bs += [tensors[f"{k}.bias"], tensors[f"{v}.bias"]]
+                bs += [tensors[f"{k}{bsf}"], tensors[f"{v}{bsf}"]]
             b_in = torch.cat([b.float() for b in bs]).contiguous()
+        if self.slope_values is not None:
+            self.slopes = torch.tensor(self.slope_values, dtype=torch.float32, device=rt.device)
         # A rotation that pairs channel j with j + rot/2: the rows of every query and key head go
         # in paired order, so that the product's kernel has both halves of a pair at hand when
         # it rotates its own result (a few decoded tokens); the rotation kernel reads that order too.
@@ -118,9 +141,9 @@ class PagedAttention(Mixer):
             if b_in is not None:
                 b_in = b_in.index_select(0, index)
         self.w_in, self.b_in = rt.ops.pack_weight(w_in), b_in
-        self.w_out = rt.ops.pack_weight(tensors[f"{o}.weight"])
+        self.w_out = rt.ops.pack_weight(tensors[f"{o}{ws}"])
         if self.out_bias:
-            self.b_out = tensors[f"{o}.bias"].float().contiguous()
+            self.b_out = tensors[f"{o}{bsf}"].float().contiguous()
 
     def _attend(self, ctx, cache, h):
         ops, rt = self.rt.ops, self.rt
@@ -153,7 +176,7 @@ class PagedAttention(Mixer):
                               rot.rotary_dim if rot else 0, rot.interleaved if rot else False,
                               rot.mscale if rot else 1.0, cache.page_size, paired=self.paired)
         return ops.attention(q, cache.k, cache.v, ctx, cache.group, H, Hk, D, cache.page_size, self.scale,
-                             self.window)
+                             self.window, slopes=self.slopes)
 
     def _step_table(self, ctx, rot):
         """The step's cosines and sines for this rotation, made once and shared by every layer
@@ -169,6 +192,9 @@ class PagedAttention(Mixer):
 
     def forward(self, ctx, cache, h):
         return self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out)
+
+    def forward_f32(self, ctx, cache, h):
+        return self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out, out_dtype=torch.float32)
 
     def forward_add(self, ctx, cache, h, residual) -> None:
         self.rt.ops.linear(self._attend(ctx, cache, h), self.w_out, bias=self.b_out, out=residual, accumulate=True)

@@ -26,6 +26,8 @@ Families and what each must offer:
   its way from the norm; ``state_spec()`` says what it carries from token to token.
 * ``Connection``: how a sublayer meets several copies of the residual stream: the weights that make its
   input of them and spread its result over them.
+* ``Injection``: ``forward(ctx, x, x0) -> x'``: remakes the 32-bit residual stream from itself and the
+  embedding's rows before the run-order entries that are entered through it.
 * ``Block``: the arrangement; it names its norms (``norm_names``), may do without a mixer or a
   feed-forward, and ``forward(ctx, cache, x)`` updates ``x`` in place.
 
@@ -57,12 +59,19 @@ class ParamSpec:
     tensors keep 32 bits if the file stores them so (bfloat16 otherwise, in a
     bfloat16 engine); "int" tensors become int32.
     ``init`` tells the random-weights mode what to write: "normal" (the model's deviation),
-    "normal:<s>" (deviation s), "ones", "ones_jitter" (1 + N(0, jitter)) or "zeros".
+    "normal:<s>" (deviation s), "ones", "ones_jitter" (1 + N(0, jitter)), "zeros", or for an integer
+    table "choice:<n>" (every row distinct numbers below n).
+    An axis of ``shape`` may be -1: a size that no configuration names and the stored tensor decides
+    (the part reads it in ``bind``); ``random_shape`` then says what the random-weights mode writes.
     """
     shape: Tuple[int, ...]
     role: str = "matrix"
     init: str = "normal"
     optional: bool = False
+    random_shape: Optional[Tuple[int, ...]] = None
+
+    def fits(self, stored: Tuple[int, ...]) -> bool:
+        return len(stored) == len(self.shape) and all(a == -1 or a == b for a, b in zip(self.shape, stored))
 
 
 @dataclass(frozen=True)
@@ -214,6 +223,18 @@ class Connection(Part):
     streams = 1
 
 
+class Injection(Part):
+    """What remakes the residual stream from itself and the embedding's rows at the start of a pass over a
+    span of layers: ``forward(ctx, x, x0) -> x'`` with ``x`` and the result 32-bit ``[T, E]``; ``x0`` is what
+    ``prepare(ctx, embedded)`` made of the embedding's rows when the step began."""
+
+    def prepare(self, ctx, embedded: torch.Tensor):
+        return embedded
+
+    def forward(self, ctx, x: torch.Tensor, x0) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class FeedForward(Part):
     def forward(self, ctx, h: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -327,7 +348,7 @@ class Runtime:
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
     "norm": {}, "position": {}, "qk_transform": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {},
-    "head": {}, "filter": {}, "connection": {},
+    "head": {}, "filter": {}, "connection": {}, "injection": {},
 }
 
 
@@ -362,6 +383,10 @@ def register_connection(kind, factory, replace=False):
     _register("connection", kind, factory, replace)
 
 
+def register_injection(kind, factory, replace=False):
+    _register("injection", kind, factory, replace)
+
+
 def register_feed_forward(kind, factory, replace=False):
     _register("feed_forward", kind, factory, replace)
 
@@ -390,12 +415,15 @@ def make_part(family: str, spec) -> Any:
     return reg[spec.kind](**spec.params)
 
 
-def make_block(kind: str, mixer, feed_forward, norms, filters=None, connections=None) -> Block:
+def make_block(kind: str, mixer, feed_forward, norms, filters=None, connections=None, params=None) -> Block:
     """The arrangement ``kind`` around the given parts (``norms``: name -> norm; ``filters``: name ->
-    sequence filter, ``connections``: name -> connection, for an arrangement that has any)."""
+    sequence filter, ``connections``: name -> connection, for an arrangement that has any; ``params``: the
+    arrangement's own constants, as keyword arguments)."""
     reg = _REGISTRIES["block"]
     if kind not in reg:
         raise ValueError(f"no block arrangement {kind!r}; registered: {sorted(reg)}")
+    if params:
+        return reg[kind](mixer, feed_forward, norms, filters or {}, connections or {}, **dict(params))
     if connections:
         return reg[kind](mixer, feed_forward, norms, filters or {}, connections)
     if filters:

@@ -14,6 +14,12 @@ without a feed-forward.
 ``x_t <- sum_s mix[s, t] x_s + out[t] y`` for all ``t`` at once, from the old copies.  ``x`` is then
 ``[S, T, E]``; the model makes the copies after the embedding and adds them up before the final norm.
 The write of one sublayer and the read and norm of the next run in one kernel.
+
+"sandwich": every sublayer is normed before and after, and what it adds is scaled:
+``x += m post_m(mixer(pre_m(x))); x += m post_f(feed_forward(pre_f(x)))`` with one number ``m`` for the
+layer.  A layer of it may come without a feed-forward.  Where all four norms are dynamic tanh, which
+takes no statistic of a row, the second norm of one sublayer, the scaled sum and the first norm of
+the next are one element-wise pass.
 """
 from __future__ import annotations
 
@@ -197,7 +203,53 @@ class StreamsPreNormBlock(Block):
         return None
 
 
+class SandwichEntry:
+    """What the block before needs to make this block's first input: its first norm."""
+
+    def __init__(self, norm):
+        self.norm = norm
+
+
+class SandwichBlock(Block):
+    chained = True
+    norm_names = ("mixer_norm", "mixer_post_norm", "feed_forward_norm", "feed_forward_post_norm")
+    needs_feed_forward = None       # with or without; the feed-forward's two norms then do nothing
+
+    def __init__(self, mixer, feed_forward, norms, filters=None, connections=None, residual_mult: float = 1.0):
+        super().__init__(mixer, feed_forward, norms, filters, connections)
+        self.residual_mult = float(residual_mult)
+
+    def entry_norm(self):
+        return SandwichEntry(self.norms["mixer_norm"])
+
+    def _add(self, ctx, x, y, post, nxt):
+        """``x += m post(y)``, then ``nxt`` of the updated rows (None: nothing comes back).  ``y`` is 32-bit."""
+        ops = ctx.ops
+        if hasattr(post, "dyt") and (nxt is None or hasattr(nxt, "dyt")):
+            dt = None
+            if nxt is not None:
+                dt = torch.float32 if getattr(nxt, "out_dtype", "compute") == "float32" else self.mixer.rt.dtype
+            return ops.dyt_step(x, y=y, post=post.dyt(), mult=self.residual_mult, norm=nxt.dyt() if nxt is not None else None,
+                                out_dtype=dt)
+        ops.add_(x, post.forward(ctx, y).contiguous(), scale=self.residual_mult)
+        return nxt.forward(ctx, x) if nxt is not None else None
+
+    def forward(self, ctx, cache, x, h=None, after=None):
+        """``h``: the result of ``mixer_norm`` if the block before made it.  ``after``: the next block's
+        ``entry_norm()``; if that block is of this arrangement too, its first input is returned."""
+        nxt = after.norm if isinstance(after, SandwichEntry) else None
+        if h is None:
+            h = self.norms["mixer_norm"].forward(ctx, x)
+        y = self.mixer.forward_f32(ctx, cache, h)
+        if self.feed_forward is None:
+            return self._add(ctx, x, y, self.norms["mixer_post_norm"], nxt)
+        h = self._add(ctx, x, y, self.norms["mixer_post_norm"], self.norms["feed_forward_norm"])
+        y = self.feed_forward.forward_f32(ctx, h)
+        return self._add(ctx, x, y, self.norms["feed_forward_post_norm"], nxt)
+
+
 register_connection("stream_connection", StreamConnection)
+register_block("sandwich", SandwichBlock)
 register_block("prenorm_streams", StreamsPreNormBlock)
 register_block("prenorm", PreNormBlock)
 register_block("prenorm_optional", PreNormOptionalBlock)

@@ -9,7 +9,11 @@ the reference does the reverse for a checkpoint that stores them fused
 
 Routed experts: ``n`` small feed-forwards ``down_e(relu(up_e(h))^2)`` of which every token uses ``top``,
 chosen by a router (32-bit logits, a softmax over all experts, the largest of score + correction;
-the weights are the chosen scores over their sum) and added up with those weights.
+the weights are the chosen scores over their sum) and added up with those weights.  Options: experts that
+are gated feed-forwards themselves, ``down_e(silu(gate_e(h)) * up_e(h))`` (``activation="swiglu"``); a choice
+without a router, by a table ``[vocab, top]`` of expert numbers that the token's id indexes, every chosen
+expert with the weight ``1 / top`` (``routing="table"``); a shared expert that runs for every token and is
+added to the sum (``shared_size``: its inner width; a gated feed-forward with the SiLU gate).
 
 Dense feed-forward: ``down(act(up(h)))`` with an activation over the whole row.  "polynorm":
 ``a N(z) + b N(z^2) + c N(z^3) + e`` with four learned numbers, powers element by element and
@@ -125,16 +129,29 @@ class DenseMLP(FeedForward):
 class RoutedExperts(FeedForward):
     """``n`` experts ``down_e(relu(up_e h)^2)`` without biases, ``top`` a token.  Tensors: ``router [n, E]``,
     ``correction [n]`` (added to the scores for the choice only), and per expert ``e<i>.up [F, E]``,
-    ``e<i>.down [E, F]``.  Nothing here reads the choice on the host: the kernels find a token's
+    ``e<i>.down [E, F]`` (gated experts: also ``e<i>.gate [F, E]``); with ``routing="table"`` no router but
+    ``table [vocab, top]`` (integers); with a shared expert ``shared.gate``, ``shared.up``, ``shared.down``.
+    Nothing here reads the choice on the host: the kernels find a token's
     experts on the device, so decode steps are recorded like any other."""
-    ACTIVATIONS = ("relu2",)
+    ACTIVATIONS = ("relu2", "swiglu")
+    ROUTINGS = ("router", "table")
     MAX_EXPERTS, MAX_TOP = 1024, 64     # MOE_MAX_EXPERTS, MOE_MAX_TOP of csrc/moe_kernels.hip
 
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, activation: str = "relu2",
                  router_name: str = "router", correction_name: str = "correction", expert_prefix: str = "e",
-                 up_name: str = "up", down_name: str = "down"):
+                 up_name: str = "up", down_name: str = "down", gate_name: str = "gate", routing: str = "router",
+                 vocab_size: int = 0, table_name: str = "table", shared_size: int = 0, shared_prefix: str = "shared."):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"routed experts: activation {activation!r} is not built (known: {list(self.ACTIVATIONS)})")
+        if routing not in self.ROUTINGS:
+            raise ValueError(f"routed experts: routing {routing!r} (known: {list(self.ROUTINGS)})")
+        if routing == "table" and int(vocab_size) < 1:
+            raise ValueError("routed experts: a table of experts by token id needs the vocabulary's size")
+        self.activation, self.routing, self.vocab_size = activation, routing, int(vocab_size)
+        self.gate_name, self.table_name = gate_name, table_name
+        self.shared = (GatedMLP(hidden_size, int(shared_size), activation="silu", gate_name=shared_prefix + "gate",
+                                up_name=shared_prefix + "up", down_name=shared_prefix + "down", weight_suffix="")
+                       if int(shared_size) > 0 else None)
         if not (1 <= int(top) <= int(num_experts)):
             raise ValueError(f"routed experts: {top} of {num_experts} experts a token")
         if int(num_experts) > self.MAX_EXPERTS or int(top) > self.MAX_TOP:       # refused when the model is built, not at its first step
@@ -147,26 +164,48 @@ class RoutedExperts(FeedForward):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E, F = self.hidden_size, self.intermediate_size
         r, c, p, u, d = self.names
-        # a router of N(0, 0.02) would score all experts alike; a correction that matters is as large as the scores differ
-        specs = {r: ParamSpec((self.num_experts, E), init="normal:0.5"),
-                 c: ParamSpec((self.num_experts,), role="vector", init="normal:0.1")}
+        if self.routing == "table":
+            specs = {self.table_name: ParamSpec((self.vocab_size, self.top), role="int", init=f"choice:{self.num_experts}")}
+        else:
+            # a router of N(0, 0.02) would score all experts alike; a correction that matters is as large as the scores differ
+            specs = {r: ParamSpec((self.num_experts, E), init="normal:0.5"),
+                     c: ParamSpec((self.num_experts,), role="vector", init="normal:0.1")}
         for e in range(self.num_experts):
+            if self.activation == "swiglu":
+                specs[f"{p}{e}.{self.gate_name}"] = ParamSpec((F, E))
             specs[f"{p}{e}.{u}"] = ParamSpec((F, E))
             specs[f"{p}{e}.{d}"] = ParamSpec((E, F))
+        if self.shared is not None:
+            specs.update(self.shared.param_specs())
         return specs
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         r, c, p, u, d = self.names
-        self.router = rt.ops.pack_weight(tensors[r])        # in the rows' dtype: the logits are a 32-bit product of the two
-        self.correction = tensors[c].float().contiguous()
-        self.w_up = torch.stack([tensors[f"{p}{e}.{u}"] for e in range(self.num_experts)]).contiguous()
+        if self.routing == "table":
+            self.table = tensors[self.table_name].to(torch.int32).contiguous()
+        else:
+            self.router = rt.ops.pack_weight(tensors[r])        # in the rows' dtype: the logits are a 32-bit product of the two
+            self.correction = tensors[c].float().contiguous()
+        if self.activation == "swiglu":     # an expert's gate rows before its up rows: one matrix [2F, E] an expert
+            self.w_up = torch.stack([torch.cat([tensors[f"{p}{e}.{self.gate_name}"], tensors[f"{p}{e}.{u}"]], dim=0)
+                                     for e in range(self.num_experts)]).contiguous()
+        else:
+            self.w_up = torch.stack([tensors[f"{p}{e}.{u}"] for e in range(self.num_experts)]).contiguous()
         self.w_down = torch.stack([tensors[f"{p}{e}.{d}"] for e in range(self.num_experts)]).contiguous()
+        if self.shared is not None:
+            self.shared.bind({name: tensors[name] for name in self.shared.param_specs()}, rt)
 
     def _run(self, ctx, h, out=None, accumulate=False):
         ops = self.rt.ops
-        idx, wts = ops.moe_route(h, self.router, self.correction, self.top)
-        return ops.moe_experts(h, self.w_up, self.w_down, idx, wts, out=out, accumulate=accumulate)
+        if self.routing == "table":
+            idx, wts = ops.table_route(self.table, ctx.token_ids, self.num_experts)
+        else:
+            idx, wts = ops.moe_route(h, self.router, self.correction, self.top)
+        out = ops.moe_experts(h, self.w_up, self.w_down, idx, wts, out=out, accumulate=accumulate, activation=self.activation)
+        if self.shared is not None:
+            self.shared.forward_add(ctx, h, out)
+        return out
 
     def forward(self, ctx, h):
         return self.rt.ops.convert(self._run(ctx, h), self.rt.dtype)

@@ -18,7 +18,16 @@ unit vectors ``x / sqrt(sum(x^2) + 1e-6)``, q also times ``D^-1/2``; ``beta = si
 S <- S + k u^T``.  The read-out is divided by its root mean square, times a weight over Dv that
 the heads share, times ``silu(Wg h)``, then ``Wo``.
 
-Both keep their projections in 32 bits from the product to the recurrence: what enters a
+``TimeMixWKV``: time mixing with a decay a token, head and key channel.  Each of r, k, v, g and the
+decay reads a mix of its own of the token's row and the row before, ``h + (h_before - h) mu_s`` (the row
+before a sequence's first is zero; the last row of a step is state).  ``r, k, v = W h_s`` (H heads of D,
+keys and values alike), ``w = exp(-exp(W2 tanh(W1 h_w) + w0))``; per head ``o = (S + diag(u) k v^T)^T r``
+from the state before the token, with the bonus ``u`` for the token itself, then ``S <- diag(w) S + k v^T``.
+Every head's read-out is divided by its root mean square, times a weight a channel of the row, times
+``silu(Wg h_g)``, then ``Wo``.  The width of ``W1``/``W2``'s inner side is no constant of a configuration:
+the stored tensors decide it.
+
+All keep their projections in 32 bits from the product to the recurrence: what enters a
 recurrence is not rounded on the way.
 """
 from __future__ import annotations
@@ -202,5 +211,81 @@ class GatedDelta(Mixer):
         self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
 
 
+class TimeMixWKV(Mixer):
+    MIXES = ("r", "k", "v", "g", "w")
+
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, eps: float, mu_prefix: str = "mu.", r_name: str = "r",
+                 k_name: str = "k", v_name: str = "v", g_name: str = "g", o_name: str = "o", w1_name: str = "w1",
+                 w2_name: str = "w2", w0_name: str = "w0", u_name: str = "u", norm_name: str = "norm"):
+        _check_sizes("wkv time mixing", num_heads, num_heads, head_dim, head_dim)
+        self.hidden_size, self.num_heads, self.head_dim, self.eps = int(hidden_size), int(num_heads), int(head_dim), float(eps)
+        self.size = self.num_heads * self.head_dim
+        self.names = dict(mu=mu_prefix, r=r_name, k=k_name, v=v_name, g=g_name, o=o_name, w1=w1_name, w2=w2_name, w0=w0_name,
+                          u=u_name, norm=norm_name)
+        self.decay_rank = 0         # the inner width of the decay's two matrices: read from the tensors
+
+    def state_spec(self):
+        from ..csrc.ops import Ops
+        D = self.head_dim
+        return {"S": StateSpec(Ops.recurrence_state_shape(self.num_heads, D, D), torch.float32),
+                "shift": StateSpec((self.hidden_size,), torch.float32)}
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, N, n = self.hidden_size, self.size, self.names
+        rank = max(4, E // 10)      # what the random-weights mode writes; a file may bring any
+        specs = {n["mu"] + s: ParamSpec((E,), role="vector", init="around:0.5:0.25") for s in self.MIXES}
+        for key in ("r", "k", "v", "g"):
+            specs[n[key]] = ParamSpec((N, E))
+        specs[n["w1"]] = ParamSpec((-1, E), random_shape=(rank, E))
+        specs[n["w2"]] = ParamSpec((N, -1), init="normal:0.3", random_shape=(N, rank))
+        # decays between 0.2 and 0.95 or so: a state that is kept for some tens of tokens, not for one and not for ever
+        specs[n["w0"]] = ParamSpec((N,), role="vector", init="around:-1.5:0.8")
+        specs[n["u"]] = ParamSpec((self.num_heads, self.head_dim), role="vector", init="normal:0.5")
+        specs[n["norm"]] = ParamSpec((N,), role="vector", init="ones_jitter")
+        specs[n["o"]] = ParamSpec((E, N))
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        n = self.names
+        w1, w2 = tensors[n["w1"]], tensors[n["w2"]]
+        if w1.shape[0] != w2.shape[1]:
+            raise ValueError(f"wkv time mixing: the decay's matrices {tuple(w1.shape)} and {tuple(w2.shape)} do not meet")
+        self.decay_rank = int(w1.shape[0])
+        self.mu = torch.stack([tensors[n["mu"] + s].float() for s in self.MIXES]).contiguous()
+        self.w_rkvg = torch.stack([tensors[n[key]] for key in ("r", "k", "v", "g")]).contiguous()      # [4, N, E]: one launch
+        self.w1, self.w2 = rt.ops.pack_weight(w1.contiguous()), rt.ops.pack_weight(w2.contiguous())
+        self.w0 = tensors[n["w0"]].float().contiguous()
+        self.u = tensors[n["u"]].float().contiguous()
+        self.w_norm = tensors[n["norm"]].float().contiguous()
+        self.w_out = rt.ops.pack_weight(tensors[n["o"]])
+
+    def _read_out(self, ctx, cache, h):
+        ops, dt = self.rt.ops, self.rt.dtype
+        E, N, H, D = self.hidden_size, self.size, self.num_heads, self.head_dim
+        if h.dtype != torch.float32:        # (a norm that rounds its rows: the mixes are then of the rounded rows)
+            h = ops.convert(h.contiguous(), torch.float32)
+        T = h.shape[0]
+        mixes = ops.token_shift(h, self.mu, cache.states["mixer.shift"], ctx, dt)          # [T, 5 E]: r, k, v, g, w
+        proj = torch.empty((T, 4 * N), dtype=torch.float32, device=h.device)
+        ops.heads_linear(mixes, self.w_rkvg, proj, 4, E, N)
+        r, k, v, gate = proj[:, :N], proj[:, N:2 * N], proj[:, 2 * N:3 * N], proj[:, 3 * N:]
+        inner = ops.linear(mixes[:, 4 * E:], self.w1, out_dtype=torch.float32)
+        ops.act_rows_(inner, "tanh")
+        x = ops.linear(inner if self.rt.is_fp32 else ops.convert(inner, dt), self.w2, bias=self.w0, out_dtype=torch.float32)
+        o = ops.linear_recurrence("wkv", r, k, v, cache.states["mixer.S"], ctx, H, H, D, D, gate=x, decay=self.u)
+        return ops.gated_rmsnorm(o, gate, self.w_norm, H, D, self.eps, dt)
+
+    def forward(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_f32(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out_dtype=torch.float32)
+
+    def forward_add(self, ctx, cache, h, residual) -> None:
+        self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
+
+
 register_mixer("retention", Retention)
+register_mixer("wkv_time_mix", TimeMixWKV)
 register_mixer("gated_delta", GatedDelta)

@@ -63,8 +63,8 @@ def check_against(expected: Mapping[str, ParamSpec], names: Iterable[str],
         if n not in have:
             continue
         shp, dt = tuple(shape_of(n)), dtype_of(n)
-        if shp != tuple(s.shape):
-            wrong.append(f"{n}: stored {list(shp)}, the model needs {list(s.shape)}")
+        if not s.fits(shp):
+            wrong.append(f"{n}: stored {list(shp)}, the model needs {list(s.shape)}" + (" (-1: any size)" if -1 in s.shape else ""))
         elif s.role == "int" and dt not in _INTS:
             wrong.append(f"{n}: stored as {dt}, the model needs an integer table")
         elif s.role != "int" and dt not in _FLOATS:

@@ -34,18 +34,28 @@ def random_tensor(name: str, spec: ParamSpec, seed: int, std: float, jitter: flo
     g = torch.Generator(device=dev)
     g.manual_seed(tensor_seed(seed, name))
     dt = torch.int32 if spec.role == "int" else (vector_dtype if spec.role == "vector" else matrix_dtype)
+    shape = tuple(spec.random_shape) if spec.random_shape is not None else tuple(spec.shape)
+    if any(a < 0 for a in shape):
+        raise ValueError(f"tensor {name}: a size the stored tensor decides needs a shape for the random-weights mode")
     if spec.init == "normal":
-        t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * std
+        t = torch.randn(shape, generator=g, dtype=torch.float32, device=dev) * std
     elif spec.init.startswith("normal:"):       # a deviation of the tensor's own, whatever the model's
-        t = torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * float(spec.init[7:])
+        t = torch.randn(shape, generator=g, dtype=torch.float32, device=dev) * float(spec.init[7:])
+    elif spec.init.startswith("around:"):       # "around:<m>:<s>": N(m, s)
+        _, m, sd = spec.init.split(":")
+        t = float(m) + torch.randn(shape, generator=g, dtype=torch.float32, device=dev) * float(sd)
+    elif spec.init.startswith("choice:"):       # an integer table: every row distinct numbers below n
+        n = int(spec.init[7:])
+        rows = int(torch.tensor(shape[:-1]).prod().item()) if len(shape) > 1 else 1
+        t = torch.stack([torch.randperm(n, generator=g, device=dev)[:shape[-1]] for _ in range(rows)]).reshape(shape)
     elif spec.init == "ones":
-        t = torch.ones(spec.shape, dtype=torch.float32, device=dev)
+        t = torch.ones(shape, dtype=torch.float32, device=dev)
     elif spec.init == "ones_jitter":
-        t = torch.ones(spec.shape, dtype=torch.float32, device=dev)
+        t = torch.ones(shape, dtype=torch.float32, device=dev)
         if jitter:
-            t = t + torch.randn(spec.shape, generator=g, dtype=torch.float32, device=dev) * jitter
+            t = t + torch.randn(shape, generator=g, dtype=torch.float32, device=dev) * jitter
     elif spec.init == "zeros":
-        t = torch.zeros(spec.shape, dtype=torch.float32, device=dev)
+        t = torch.zeros(shape, dtype=torch.float32, device=dev)
     else:
         raise ValueError(f"tensor {name}: unknown init {spec.init!r}")
     return t.to(dt)
