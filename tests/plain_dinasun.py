@@ -154,8 +154,8 @@ def forward(cfg, w, tokens, layers_out=None):
     """Logits ``[T, vocab]`` of the whole sequence.  ``layers_out``: a list that receives the residual
     stream after every layer run."""
     eps = cfg["norm"]["eps"]
-    mult = cfg["residual_mult"]
-    x = w["embed"][np.asarray(tokens, dtype=np.int64)] * cfg["embedding"]["scale"]
+    mult = cfg.get("residual_mult", 1.0)
+    x = w["embed"][np.asarray(tokens, dtype=np.int64)] * (cfg.get("embedding") or {}).get("scale", 1.0)
     x0 = x
     for i, enters in run_order(cfg):
         layer, p = cfg["layers"][i], f"l{i}."
