@@ -106,11 +106,14 @@ TINY_D6 = {
     ],
 }
 
-CONFIGS = {"D1": (TINY_D1, 31), "D2": (TINY_D2, 32), "D3": (TINY_D3, 33), "D4": (TINY_D4, 34), "D5": (TINY_D5, 35),
-           "D6": (TINY_D6, 36)}
+# (configuration, seed, deviation of the matrices: smaller where a factor above one and two passes over the
+# whole model would otherwise make single rows pass a rounding on a hundredfold, in 32 bits as in 16)
+CONFIGS = {"D1": (TINY_D1, 31, 0.2), "D2": (TINY_D2, 32, 0.2), "D3": (TINY_D3, 33, 0.1), "D4": (TINY_D4, 34, 0.2),
+           "D5": (TINY_D5, 35, 0.2), "D6": (TINY_D6, 36, 0.2)}
 
 
-def make_model(which: str, folder: str, std: float = 0.2) -> str:
+def make_model(which: str, folder: str, std: float = 0.0) -> str:
     from xyntetik_runner_amd.weights import write_random_model
-    config, seed = CONFIGS[which]
+    config, seed, own = CONFIGS[which]
+    std = std or own
     return write_random_model(config, folder, seed=seed, std=std, norm_jitter=0.1, dtype="bfloat16")

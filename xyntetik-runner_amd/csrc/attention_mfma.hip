@@ -64,6 +64,7 @@ struct AttnArgs {
     int n_items, n_cta_items, H, Hk, page_shift, page_mask, page_size;
     float scale;
     int window;
+    const float* slopes;    // [H], or null: slopes[h] * (i - j) is taken off the score of query i and key j
 };
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
@@ -107,6 +108,23 @@ __device__ inline float max_across_halves(float x) {
     float o;
     asm("v_max_f32 %0, %1, %2" : "=v"(o) : "v"(__uint_as_float(r[0])), "v"(__uint_as_float(r[1])));
     return o;
+}
+// What the score product of a tile starts from in the lane's row: zero, or, with distance slopes, the row's
+// bias over the tile's keys in units of the scale, (slope_h / scale) * (key - pos), so that the product's sum
+// times the scale is the biased score and the softmax below needs to know nothing of it.  (Far keys make the
+// sum large and coarse, and have no weight; the row's own key, at distance 0, is always among the visible.)
+template <bool SLOPES>
+__device__ __forceinline__ f32x16 score_start(float sb, int kt, int lg, int pos) {
+    f32x16 z;
+    if constexpr (SLOPES) {
+        const float tb = sb * (float)(kt + 8 * lg - pos);
+#pragma unroll
+        for (int e = 0; e < 16; ++e) z[e] = fmaf(sb, (float)(16 * (e >> 3) + (e & 7)), tb);
+    } else {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) z[e] = 0.f;
+    }
+    return z;
 }
 #define MAX_SLACK 8.0f
 #define ATTN_SOFTMAX_STEP(KT, KEND)                                                                  \
@@ -262,6 +280,7 @@ struct CtaWave {
     uint32_t vbase[2];          // and of its V^T fragments of channels 0-31, keys 0-15 and 16-31
     bf16x8 qf[KD];
     float c2;
+    float sb;                   // the row's head's slope over the scale (0 without slopes)
     int pos, lo, lg;
     bool row_ok;
     int kbeg, kend, nt, seq_len;
@@ -314,11 +333,11 @@ struct CtaFrags {
     }
 };
 
-template <int STAGE>
+template <int STAGE, bool SLOPES>
 __device__ __forceinline__ void cta_step_whole(const CtaWave& w, int v, f32x16& s_new, const f32x16& s_cur,
                                                uint4 (&pf_new)[2], const uint4 (&pf_old)[2], f32x16 (&o)[DB], float& m, float& l) {
     constexpr int NS = KD + 2 * DB, AHEAD = 3 < NS ? 3 : NS;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const f32x16 start = score_start<SLOPES>(w.sb, w.kbeg + v * 32, w.lg, w.pos);
     const CtaFrags f(w, v, std::integral_constant<int, STAGE>{});
     const f32x16& s = s_cur;
     uint4 fr[NS];
@@ -329,7 +348,7 @@ __device__ __forceinline__ void cta_step_whole(const CtaWave& w, int v, f32x16& 
     static_for<0, NS>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         if constexpr (k + AHEAD < NS) fr[k + AHEAD] = f.template get<k + AHEAD>();
-        if constexpr (k == 0) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), w.qf[k], zero, 0, 0, 0);
+        if constexpr (k == 0) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), w.qf[k], start, 0, 0, 0);
         else if constexpr (k < KD) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(fr[k]), w.qf[k], s_new, 0, 0, 0);
         else {
             constexpr int j = (k - KD) / DB, d = (k - KD) % DB;
@@ -377,17 +396,16 @@ __device__ __forceinline__ void cta_step_whole(const CtaWave& w, int v, f32x16& 
     }
 }
 
-template <int STAGE>
+template <int STAGE, bool SLOPES>
 __device__ __forceinline__ void cta_step_edge(const CtaWave& w, int v, f32x16& s_new, const f32x16& s_cur,
                                               uint4 (&pf_new)[2], const uint4 (&pf_old)[2], f32x16 (&o)[DB], float& m, float& l) {
     constexpr int NS = KD + 2 * DB;
-    const f32x16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const CtaFrags f(w, v, std::integral_constant<int, STAGE>{});
     const int lg = w.lg;
     if (w.sees(v)) {
         uint4 kf[KD];
         static_for<0, KD>([&](auto kc) { kf[decltype(kc)::value] = f.template get<decltype(kc)::value>(); });
-        s_new = zero;
+        s_new = score_start<SLOPES>(w.sb, w.kbeg + v * 32, w.lg, w.pos);
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) s_new = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), w.qf[kd], s_new, 0, 0, 0);
     }
@@ -433,6 +451,7 @@ __device__ __forceinline__ void cta_step_edge(const CtaWave& w, int v, f32x16& s
 }
 
 // The kernel.  A place of the ring holds K of tile v beside V^T of tile v-2, which is what step v reads.
+template <bool SLOPES>
 __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
     using SH = CtaShape;
     constexpr int SET_THREADS = SH::SET_THREADS, LOADS = SH::LOADS, STAGE = SH::STAGE, SETS = SH::SETS;
@@ -472,6 +491,7 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
         w.pos = start + tok;
         w.lo = (a.window > 0 && w.pos - a.window + 1 > 0) ? w.pos - a.window + 1 : 0;
         w.lg = lg;
+        w.sb = SLOPES ? a.slopes[kvh * G + hg] / a.scale : 0.f;
         const bf16_t* qp = a.q + ((size_t)(row_ok ? it[5] + tok : it[5]) * a.H + kvh * G + hg) * HD + lg * 8;
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd) w.qf[kd] = as_bf16x8(keep_if(row_ok, ldg16(qp + kd * 16)));
@@ -647,18 +667,18 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
     int v = 0;
     for (; v < v1; v += 2) {
         STEPS_SYNC(v)
-        cta_step_edge<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
-        cta_step_edge<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+        cta_step_edge<STAGE, SLOPES>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_edge<STAGE, SLOPES>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
     }
     for (; v < v2; v += 2) {
         STEPS_SYNC(v)
-        cta_step_whole<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
-        cta_step_whole<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+        cta_step_whole<STAGE, SLOPES>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_whole<STAGE, SLOPES>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
     }
     for (; v < n_steps; v += 2) {
         STEPS_SYNC(v)
-        cta_step_edge<STAGE>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
-        cta_step_edge<STAGE>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
+        cta_step_edge<STAGE, SLOPES>(w, v, s_even, s_odd, pf_odd, pf_even, o, m, l);
+        cta_step_edge<STAGE, SLOPES>(w, v + 1, s_odd, s_even, pf_even, pf_odd, o, m, l);
     }
 #undef STEPS_SYNC
 #undef STEPS_ISSUE
@@ -741,6 +761,7 @@ constexpr int STREAM_LDS_BYTES = STREAM_RING_BYTES > STREAM_MERGE_BYTES ? STREAM
 static_assert(W_LOADS * (STREAM_STAGES - 1) < 64, "too many copies in flight for the counter");
 static_assert(STREAM_LDS_BYTES <= 160 * 1024, "the rings do not fit into LDS");
 
+template <bool SLOPES>
 __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     extern __shared__ uint4 lds[];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -765,6 +786,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     const int t = q0 + tok, h = kvh * G + hg;
     const int pos = start + tok;
     const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+    const float sb = SLOPES ? a.slopes[h] / a.scale : 0.f;
 
     bf16x8 qf[KD];
     {
@@ -899,9 +921,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
                 }
             }
         }
-        f32x16 s;
-#pragma unroll
-        for (int e = 0; e < 16; ++e) s[e] = 0.f;
+        f32x16 s = score_start<SLOPES>(sb, kt, lg, pos);
 #pragma unroll
         for (int kd = 0; kd < KD; ++kd)
             s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(kf[kd]), qf[kd], s, 0, 0, 0);
@@ -1047,7 +1067,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
                                  const int* cu_q,
                                  const int* starts, const int* block_table, int table_stride, float* part_o,
                                  float* part_ml, int H, int Hk, int D, int page_size, float scale, int window,
-                                 hipStream_t stream) {
+                                 const float* slopes, hipStream_t stream) {
     XR_REQUIRE(D == HD, "attention: this library is compiled for head size %d, got %d", HD, D);
     XR_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
     int shift = ilog2_exact(page_size);
@@ -1064,28 +1084,33 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     a.cta_items = items; a.n_cta_items = n_cta_items; a.items = items + (size_t)n_cta_items * ITEM_INTS; a.cu_q = cu_q; a.starts = starts; a.block_table = block_table; a.table_stride = table_stride;
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
+    a.slopes = slopes;
+    XR_REQUIRE(!slopes || scale > 0.f, "attention: distance slopes need a positive scale, got %g", (double)scale);
     if (n_cta_items > 0) {
         constexpr int smem = CtaShape::LDS_BYTES;
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void*)k_attn_cta, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        static bool attr_set[2] = {false, false};
+        const void* kernel = slopes ? (const void*)k_attn_cta<true> : (const void*)k_attn_cta<false>;
+        if (!attr_set[slopes != nullptr]) {
+            hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             if (e != hipSuccess) (void)hipGetLastError();     // or the next launch's check would report this refusal
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", smem, hipGetErrorString(e));
-            attr_set = true;
+            attr_set[slopes != nullptr] = true;
         }
-        k_attn_cta<<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape::THREADS, smem, stream>>>(a);
+        if (slopes) k_attn_cta<true><<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape::THREADS, smem, stream>>>(a);
+        else k_attn_cta<false><<<dim3((unsigned)n_cta_items * (unsigned)Hk), CtaShape::THREADS, smem, stream>>>(a);
         XR_CHECK_LAUNCH("attention_cta");
     }
     if (n_items > 0) {
-        static bool attr_set = false;
-        if (!attr_set) {
-            hipError_t e = hipFuncSetAttribute((const void*)k_attn_stream, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                               STREAM_LDS_BYTES);
+        static bool attr_set[2] = {false, false};
+        const void* kernel = slopes ? (const void*)k_attn_stream<true> : (const void*)k_attn_stream<false>;
+        if (!attr_set[slopes != nullptr]) {
+            hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, STREAM_LDS_BYTES);
             if (e != hipSuccess) (void)hipGetLastError();
             XR_REQUIRE(e == hipSuccess, "attention: %d bytes of LDS refused: %s", STREAM_LDS_BYTES, hipGetErrorString(e));
-            attr_set = true;
+            attr_set[slopes != nullptr] = true;
         }
-        k_attn_stream<<<dim3((unsigned)n_items * (unsigned)Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
+        if (slopes) k_attn_stream<true><<<dim3((unsigned)n_items * (unsigned)Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
+        else k_attn_stream<false><<<dim3((unsigned)n_items * (unsigned)Hk), 64 * STREAM_WAVES, STREAM_LDS_BYTES, stream>>>(a);
         XR_CHECK_LAUNCH("attention_stream");
     }
     if (n_jobs > 0) {

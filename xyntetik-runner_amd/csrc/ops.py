@@ -614,8 +614,7 @@ class Ops:
             self._dev(slopes)
             if slopes.dtype != torch.float32 or slopes.numel() != H or not slopes.is_contiguous():
                 raise KernelError(f"attention: the slopes must be float32 [{H}]")
-        if (self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16
-                and slopes is None):
+        if self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16:
             lib = self.attention_lib(D)
             plan = ctx.attention_plan(group, H // Hk, window, Hk, page_size)
             part_o = part_ml = None
@@ -626,7 +625,7 @@ class Ops:
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(window or 0), _stream()))
+                float(scale), int(window or 0), _ptr(slopes), _stream()))
             return out
         self.lib.check(self.lib.xr_attention_ref(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
@@ -641,7 +640,7 @@ class Ops:
             unit = f"attn_d{D}"
             path = _build.find_built(unit) or _build.build_unit(unit)
             lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _p, _p,
-                                                    _i, _i, _i, _i, _f, _i, _p]})
+                                                    _i, _i, _i, _i, _f, _i, _p, _p]})
             self._attn_libs[D] = lib
         return lib
 
@@ -1223,7 +1222,7 @@ class Ops:
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), table.data_ptr(), table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(size), _stream()))
+                float(scale), int(size), None, _stream()))
             return out
         self.lib.check(self.lib.xr_attention_pooled(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(pk) if P else None,
