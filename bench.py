@@ -328,7 +328,27 @@ def sugosun_config(width, layers, vocab=32000):
             "embedding": {"bigram": {"buckets": 100003, "mul_prev": 1000003, "mul_cur": 999983}}, "layers": out}
 
 
-DESIGNS = {"suripel": ("Suripel", suripel_config), "sugosun": ("Sugosun", sugosun_config)}
+def dinasun_config(width, layers, vocab=32000):
+    """A Dinasun model of real layer sizes whose layer runs are ``layers``: time mixing with heads of 64 and
+    attention with heads of 128 (four query heads a key/value head, a temperature step every 1,024 positions) in
+    turn, every layer with 16 gated experts of width / 2 (2 a token, by the table) and a shared expert of the
+    model's width; a third of the runs are the second pass over a span in the middle."""
+    again = layers // 3
+    distinct = layers - again
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 16, "top": 2}, "shared": {"ff": width}}
+    H = width // 128
+    wkv = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64}, "mlp": moe}
+    att = {"type": "attention", "mixer": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                          "q_temp": {"coef": 0.1, "every": 1024}}, "mlp": moe}
+    cfg = {"architecture": "Dinasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+           "embedding": {"scale": 1.0}, "layers": [wkv if i % 2 == 0 else att for i in range(distinct)]}
+    if again:
+        start = (distinct - again) // 2
+        cfg["loop"] = {"start": start, "stop": start + again, "times": 2}
+    return cfg
+
+
+DESIGNS = {"suripel": ("Suripel", suripel_config), "sugosun": ("Sugosun", sugosun_config), "dinasun": ("Dinasun", dinasun_config)}
 
 
 def llama_like(width, layers, vocab=32000):
@@ -431,7 +451,7 @@ def main():
                     help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
-    ap.add_argument("--design", default="", choices=["", "suripel", "sugosun"],
+    ap.add_argument("--design", default="", choices=["", "suripel", "sugosun", "dinasun"],
                     help="instead of the serving benchmark: this design at real layer sizes beside the Llama decoder of equal size")
     ap.add_argument("--design-sizes", default="2048,4096", metavar="LIST", help="widths of the --design models")
     ap.add_argument("--design-layers", type=int, default=12, help="layers of the --design models")

@@ -171,12 +171,57 @@ def test_wkv_recurrence_in_portions(ops, H, D):
         close(got[r], want[r], 5e-6, f"request {r}")
 
 
-def test_a_far_write_is_kept_by_a_channel_that_does_not_decay(ops):
-    """Token 2 writes a value along key channel 0 (decay exp(-exp(-30)) = 1) and another along channel 1
-    (decay exp(-exp(1)) = 0.07): 600 tokens later a query on channel 0 returns the first whole, a query on
-    channel 1 nothing.  The bonus enters the token's own read-out and is not written into the state."""
+@pytest.mark.parametrize("H,D", [(2, 64), (3, 16), (1, 40)])
+def test_wkv_recurrence_over_long_portions(ops, H, D):
+    """Portions from 1,024 rows on run as chunks side by side: a chunk's last state from zero plus the state
+    before it times the product of the chunk's decays, channel by channel.  Three requests in one step (a long
+    portion that ends inside a chunk, a short one, one of exactly four chunks), then their rest from the
+    states that the chunks left; decays from 0.69 to 0.9975, so that a chunk's first state still counts at its end."""
     from xyntetik_runner_amd.csrc.ops import Ops
-    H, D, n = 2, 12, 610
+    rng = np.random.default_rng(H + D)
+    lens = [1300, 40, 2100]
+    N = H * D
+    rows = [rng.normal(size=(L, 4 * N)) for L in lens]
+    for x in rows:
+        x[:, N:2 * N] *= 0.3
+        x[:, 3 * N:] = rng.uniform(-6.0, -1.0, size=(x.shape[0], N))
+    u = rng.normal(size=(H, D)) * 0.5
+    want = []
+    for x in rows:
+        L = x.shape[0]
+        r, k, v = (x[:, i * N:(i + 1) * N].reshape(L, H, D) for i in range(3))
+        decay = np.exp(-np.exp(x[:, 3 * N:])).reshape(L, H, D)
+        want.append(np.stack([P.wkv_recurrence(r[:, i], k[:, i], v[:, i], decay[:, i], u[i]) for i in range(H)], axis=1).reshape(L, N))
+    state = torch.full((5,) + Ops.recurrence_state_shape(H, D, D), float("nan"), device=DEV)
+    slots = [4, 0, 2]
+    for sl in slots:
+        state[sl] = 0.0
+    got = [np.zeros_like(w) for w in want]
+    at = [0, 0, 0]
+    for takes in ([1100, 40, 1024], [200, 0, 1076]):
+        live = [r for r in range(3) if takes[r] > 0]
+        ctx = step_ctx([at[r] for r in live], [takes[r] for r in live], [slots[r] for r in live])
+        row = dev(np.concatenate([rows[r][at[r]:at[r] + takes[r]] for r in live]))
+        o = ops.linear_recurrence("wkv", row[:, :N], row[:, N:2 * N], row[:, 2 * N:3 * N], state, ctx, H, H, D, D,
+                                  gate=row[:, 3 * N:].contiguous(), decay=dev(u)).cpu().numpy()
+        k = 0
+        for r in live:
+            got[r][at[r]:at[r] + takes[r]] = o[k:k + takes[r]]
+            k += takes[r]
+            at[r] += takes[r]
+    assert at == lens
+    for r in range(3):
+        close(got[r], want[r], 2e-5, f"request {r}")
+    assert torch.isnan(state[1]).all() and torch.isnan(state[3]).all()
+
+
+@pytest.mark.parametrize("n,sizes", [(610, [40, 1, 1, 300, 2, 1]), (2700, [1500, 1, 1100, 2])])
+def test_a_far_write_is_kept_by_a_channel_that_does_not_decay(ops, n, sizes):
+    """Token 2 writes a value along key channel 0 (decay exp(-exp(-30)) = 1) and another along channel 1
+    (decay exp(-exp(1)) = 0.07): 600 tokens later (or 2,700, across chunks) a query on channel 0 returns the
+    first whole, a query on channel 1 nothing.  The bonus enters the token's own read-out and is not written into the state."""
+    from xyntetik_runner_amd.csrc.ops import Ops
+    H, D = 2, 12
     N = H * D
     rng = np.random.default_rng(8)
     r = np.zeros((n, H, D)); k = rng.normal(size=(n, H, D)) * 0.01; v = rng.normal(size=(n, H, D))
@@ -195,7 +240,7 @@ def test_a_far_write_is_kept_by_a_channel_that_does_not_decay(ops):
     state = torch.full((3,) + Ops.recurrence_state_shape(H, D, D), float("nan"), device=DEV)
     state[1] = 0.0
     got = np.zeros((n, H, D))
-    for i, m in cuts(n, [40, 1, 1, 300, 2, 1]):
+    for i, m in cuts(n, sizes):
         ctx = step_ctx([i], [m], [1])
         row = dev(np.concatenate([a[i:i + m].reshape(m, -1) for a in (r, k, v, x)], axis=1))
         o = ops.linear_recurrence("wkv", row[:, :N], row[:, N:2 * N], row[:, 2 * N:3 * N], state, ctx, H, H, D, D,

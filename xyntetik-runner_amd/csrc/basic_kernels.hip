@@ -176,21 +176,60 @@ __global__ __launch_bounds__(256) void k_dyt_step(DytArgs a) {
     const int c = (int)(i - r * per_row) * NV;
     const size_t src = a.rows ? (size_t)a.rows[r] : r;
     float* xp = a.x + src * a.ldx + c;
-    float v[NV];
+    float v[NV], wv[NV], bv[NV];
+    // NV = 4: E, ldx and c are multiples of 4 and the tensors' starts are 16-byte aligned, so a lane's four
+    // values are one load and one store
+    if constexpr (NV == 4) {
+        const float4 t = *reinterpret_cast<const float4*>(xp);
+        v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w;
+    } else {
 #pragma unroll
-    for (int k = 0; k < NV; ++k) v[k] = xp[k];
+        for (int k = 0; k < NV; ++k) v[k] = xp[k];
+    }
+    auto vec = [&](const float* p, float (&o)[NV]) {
+        if constexpr (NV == 4) {
+            const float4 t = *reinterpret_cast<const float4*>(p + c);
+            o[0] = t.x; o[1] = t.y; o[2] = t.z; o[3] = t.w;
+        } else {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) o[k] = p[c + k];
+        }
+    };
     if (a.y) {
+        float yv[NV];
+        if constexpr (NV == 4 && sizeof(TY) == 4) {
+            const float4 t = *reinterpret_cast<const float4*>((const float*)a.y + r * a.E + c);
+            yv[0] = t.x; yv[1] = t.y; yv[2] = t.z; yv[3] = t.w;
+        } else if constexpr (NV == 4) {
+            const uint2 t = *reinterpret_cast<const uint2*>((const bf16_t*)a.y + r * a.E + c);
+            yv[0] = __uint_as_float(t.x << 16); yv[1] = __uint_as_float(t.x & 0xffff0000u);
+            yv[2] = __uint_as_float(t.y << 16); yv[3] = __uint_as_float(t.y & 0xffff0000u);
+        } else {
 #pragma unroll
-        for (int k = 0; k < NV; ++k) {
-            const float yv = ld<TY>((const TY*)a.y, r * a.E + c + k);
-            v[k] = v[k] + a.mult * fmaf(tanhf(a.alpha_p * yv), a.w_p[c + k], a.b_p[c + k]);
-            xp[k] = v[k];
+            for (int k = 0; k < NV; ++k) yv[k] = ld<TY>((const TY*)a.y, r * a.E + c + k);
+        }
+        vec(a.w_p, wv); vec(a.b_p, bv);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) v[k] = v[k] + a.mult * fmaf(tanhf(a.alpha_p * yv[k]), wv[k], bv[k]);
+        if constexpr (NV == 4) *reinterpret_cast<float4*>(xp) = make_float4(v[0], v[1], v[2], v[3]);
+        else {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) xp[k] = v[k];
         }
     }
     if (a.h) {
+        vec(a.w_n, wv); vec(a.b_n, bv);
+        float o[NV];
 #pragma unroll
-        for (int k = 0; k < NV; ++k)
-            st<TO>((TO*)a.h, r * a.E + c + k, fmaf(tanhf(a.alpha_n * v[k]), a.w_n[c + k], a.b_n[c + k]));
+        for (int k = 0; k < NV; ++k) o[k] = fmaf(tanhf(a.alpha_n * v[k]), wv[k], bv[k]);
+        if constexpr (NV == 4 && sizeof(TO) == 4)
+            *reinterpret_cast<float4*>((float*)a.h + r * a.E + c) = make_float4(o[0], o[1], o[2], o[3]);
+        else if constexpr (NV == 4)
+            *reinterpret_cast<uint2*>((bf16_t*)a.h + r * a.E + c) = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+        else {
+#pragma unroll
+            for (int k = 0; k < NV; ++k) st<TO>((TO*)a.h, r * a.E + c + k, o[k]);
+        }
     }
 }
 
@@ -205,7 +244,8 @@ extern "C" int xr_dyt_step(float* x, const void* y, const float* w_p, const floa
     XR_REQUIRE((y_dtype == XR_F32 || y_dtype == XR_BF16) && (h_dtype == XR_F32 || h_dtype == XR_BF16),
                "dyt: bad dtypes y=%d h=%d", y_dtype, h_dtype);
     if (R == 0) return XR_OK;
-    const bool vec = E % 4 == 0 && ldx % 4 == 0;
+    auto al16 = [](const void* p) { return p == nullptr || (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    const bool vec = E % 4 == 0 && ldx % 4 == 0 && al16(x) && al16(y) && al16(h) && al16(w_p) && al16(b_p) && al16(w_n) && al16(b_n);
     DytArgs a{x, y, w_p, b_p, alpha_p, mult, h, w_n, b_n, alpha_n, rows, E, ldx, (size_t)R * (E / (vec ? 4 : 1))};
     const unsigned blocks = (unsigned)((a.n + 255) / 256);
 #define DY(TY, TO)                                                                  \

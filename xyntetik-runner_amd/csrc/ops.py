@@ -82,7 +82,7 @@ _PROTOS = {
     "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
     "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
-    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _i, _p],
+    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_attention_pool_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
@@ -1137,19 +1137,22 @@ class Ops:
         elif decay is None or decay.dtype != torch.float32 or decay.numel() != H:
             raise KernelError(f"linear_recurrence: retention needs float32 decay [{H}]")
         out = torch.empty((T, H * Dv), dtype=torch.float32, device=q.device)
-        # Retention over long portions runs in chunks side by side (its decay is one number a head, so a
-        # chunk's sum from zero and the decayed state before it add up); the delta rule's chain cannot be cut.
-        chunk_len, n_chunks, scratch = 0, 0, None
-        if kind == "retention" and ctx.max_q_len >= self.RETENTION_CHUNKED_FROM:
+        # Retention and wkv over long portions run in chunks side by side (the state before a chunk enters the
+        # chunk's last state through the chunk's decays alone: one number a head, or their product channel by
+        # channel; a chunk's sum from zero and that add up); the delta rule's chain cannot be cut.
+        chunk_len, n_chunks, scratch, prod = 0, 0, None, None
+        if kind in ("retention", "wkv") and ctx.max_q_len >= self.RETENTION_CHUNKED_FROM:
             n = -(-ctx.max_q_len // self.RETENTION_CHUNK)
             if ctx.B * n <= 4096:
                 chunk_len, n_chunks = self.RETENTION_CHUNK, n
                 scratch = torch.empty((ctx.B * n,) + tuple(state.shape[1:]), dtype=torch.float32, device=q.device)
+                if kind == "wkv":
+                    prod = torch.empty((ctx.B * n, H, rows.value * lanes.value), dtype=torch.float32, device=q.device)
         self.lib.check(self.lib.xr_linear_recurrence(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(beta),
                                                      _ptr(gate), _ptr(decay), state.data_ptr(), ctx.cu_q.data_ptr(),
                                                      ctx.slots.data_ptr(), ctx.B, H, G, D, Dv, q.stride(0),
                                                      gates[0].stride(0) if gates else 0, RECURRENCES[kind],
-                                                     chunk_len, n_chunks, _ptr(scratch), 1 if activation else 0, _stream()))
+                                                     chunk_len, n_chunks, _ptr(scratch), _ptr(prod), 1 if activation else 0, _stream()))
         return out
 
     RETENTION_CHUNK = 256            # rows a chunk; a multiple of the kernel's 16 staged tokens

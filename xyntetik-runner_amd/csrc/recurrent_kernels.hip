@@ -51,6 +51,11 @@ struct RecArgs {
     int pass, chunk_len, n_chunks;
     float* scratch;
     int act;                 // 1: q, k and v pass SiLU as they are fetched (0: they are taken as they are)
+    // wkv in chunks: its decay is a number a token and key channel, so the state before a chunk enters the
+    // chunk's last state through the product of the chunk's decays, channel by channel: pass 1 leaves that
+    // product in prod [request x chunk][head][J][R] (row R j + r at j R + r) beside the chunk's last state;
+    // pass 2 runs with v = 0, so that the state only decays and the bonus term is nothing.
+    float* prod;
 };
 
 // the value of lane (l ^ 1), (l ^ 2) of a quad, or of the lane 4 / 8 further round a row of 16
@@ -79,7 +84,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
     const int cl = tid / R, r = tid % R;
     const int col = blockIdx.x * COLS + cl;
     const bool live = col < a.Dv;
-    const int pass = MODE == XR_REC_RETENTION ? a.pass : 0;
+    const int pass = MODE != XR_REC_DELTA ? a.pass : 0;
     int b = blockIdx.z, chunk = 0;
     if (pass) { chunk = b % a.n_chunks; b /= a.n_chunks; }
     int row0 = a.cu_q[b], n = a.cu_q[b + 1] - row0;
@@ -102,8 +107,13 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
     float* kf = reinterpret_cast<float*>(&ks[0][0]);
     float* wf = reinterpret_cast<float*>(&ws[0][0]);
     float ub[DPER];                 // (wkv) the bonus of this lane's rows
+    float wp[MODE == XR_REC_WKV ? DPER : 1];        // (wkv, pass 1) the product of the chunk's decays of this lane's rows
 #pragma unroll
     for (int j = 0; j < DPER; ++j) ub[j] = (MODE == XR_REC_WKV && R * j + r < a.D) ? a.decay[(size_t)h * a.D + R * j + r] : 0.f;
+    if (MODE == XR_REC_WKV) {
+#pragma unroll
+        for (int j = 0; j < DPER; ++j) wp[j] = 1.f;
+    }
 
     // A chunk's queries, keys, values and gates go from memory into registers while the chunk before
     // it is computed, and from there into LDS: the chain of tokens never waits for memory.
@@ -205,6 +215,7 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
                     o0 = fmaf(q4.z, fmaf(ub[j + 2], t2, S[j + 2]), o0); o1 = fmaf(q4.w, fmaf(ub[j + 3], t3, S[j + 3]), o1);
                     S[j] = fmaf(w4.x, S[j], t0); S[j + 1] = fmaf(w4.y, S[j + 1], t1);
                     S[j + 2] = fmaf(w4.z, S[j + 2], t2); S[j + 3] = fmaf(w4.w, S[j + 3], t3);
+                    if (pass == 1) { wp[j] *= w4.x; wp[j + 1] *= w4.y; wp[j + 2] *= w4.z; wp[j + 3] *= w4.w; }
                 }
                 return o0 + o1;
             };
@@ -217,12 +228,18 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
                 for (int x = 0; x < 4; ++x) oo[x] = group_sum<R>(oo[x]);
                 if (live && r == 0) {
 #pragma unroll
-                    for (int x = 0; x < 4; ++x) a.out[((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col] = oo[x];
+                    for (int x = 0; x < 4; ++x) {
+                        float* dst = a.out + ((size_t)(row0 + c0 + tt + x) * a.H + h) * a.Dv + col;
+                        *dst = pass == 2 ? *dst + oo[x] : oo[x];
+                    }
                 }
             }
             for (; tt < nt; ++tt) {
                 const float o = group_sum<R>(token(tt));
-                if (live && r == 0) a.out[((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col] = o;
+                if (live && r == 0) {
+                    float* dst = a.out + ((size_t)(row0 + c0 + tt) * a.H + h) * a.Dv + col;
+                    *dst = pass == 2 ? *dst + o : o;
+                }
             }
         } else {
             // Retention's chain is one multiply-add a token; four tokens' read-outs run side by side.
@@ -292,27 +309,37 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
         for (int j = 0; j < DPER; ++j)
             if (j < J) to[((size_t)j * a.Dv + col) * R + r] = S[j];
     }
+    if (MODE == XR_REC_WKV && pass == 1 && col == 0) {      // every column holds the same products: the first writes them
+        float* pp = a.prod + (((size_t)b * a.n_chunks + chunk) * a.H + h) * J * R;
+#pragma unroll
+        for (int j = 0; j < DPER; ++j)
+            if (j < J) pp[j * R + r] = wp[j];
+    }
 }
 
 // Between the two passes over the chunks: scratch[b][c] holds chunk c's last state as if it had begun at
 // zero (chunk 0's is true).  In place, chunk by chunk: the true first state of chunk c (for pass 2), and
 // at the end the request's new state.  One thread an element of a head's state.
-__global__ __launch_bounds__(256) void k_retention_carry(RecArgs a, int per_head) {
+template <bool WKV>
+__global__ __launch_bounds__(256) void k_retention_carry(RecArgs a, int per_head, int R) {
     const int b = blockIdx.z, h = blockIdx.y;
     const int e = blockIdx.x * 256 + threadIdx.x;
     if (e >= per_head) return;
     const int n = a.cu_q[b + 1] - a.cu_q[b];
     if (n <= 0) return;
     const int nc = (n + a.chunk_len - 1) / a.chunk_len;
-    const float dec = a.decay[h];
+    const float dec = WKV ? 1.f : a.decay[h];
     const size_t step = (size_t)a.H * per_head;
     float* cp = a.scratch + ((size_t)b * a.n_chunks * a.H + h) * per_head + e;
+    // (wkv) element e = (j Dv + c) R + r of the state is row R j + r, whose product lies at j R + r
+    const int JR = per_head / a.Dv;
+    const float* pp = WKV ? a.prod + ((size_t)b * a.n_chunks * a.H + h) * JR + (e / (a.Dv * R)) * R + e % R : nullptr;
     float t = cp[0];
     for (int c = 1; c < nc; ++c) {
         const int len = n - c * a.chunk_len < a.chunk_len ? n - c * a.chunk_len : a.chunk_len;
         const float own = cp[c * step];
         cp[c * step] = t;
-        t = fmaf(powf(dec, (float)len), t, own);
+        t = fmaf(WKV ? pp[(size_t)c * a.H * JR] : powf(dec, (float)len), t, own);
     }
     a.state[((size_t)a.slots[b] * a.H + h) * per_head + e] = t;
 }
@@ -327,7 +354,7 @@ extern "C" int xr_recurrence_state_dims(int D, int* rows, int* lanes) {
 extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, const float* v, const float* beta,
                                     const float* gate, const float* decay, float* state, const int* cu_q,
                                     const int* slots, int B, int H, int G, int D, int Dv, int ld, int ld_g, int mode,
-                                    int chunk_len, int n_chunks, float* scratch, int act, hipStream_t stream) {
+                                    int chunk_len, int n_chunks, float* scratch, float* prod, int act, hipStream_t stream) {
     XR_REQUIRE(B >= 0 && H > 0 && G > 0 && H % G == 0, "recurrence: %d heads over %d key heads", H, G);
     XR_REQUIRE(D > 0 && D <= 256 && Dv > 0, "recurrence: key size %d (1 to 256), value size %d", D, Dv);
     XR_REQUIRE(mode == XR_REC_RETENTION || mode == XR_REC_DELTA || mode == XR_REC_WKV, "recurrence: mode %d", mode);
@@ -339,10 +366,11 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
     XR_REQUIRE(act == 0 || act == 1, "recurrence: activation %d of q, k and v (0: none, 1: SiLU)", act);
     if (B == 0) return XR_OK;
     const bool chunks = chunk_len > 0;
-    XR_REQUIRE(!chunks || (mode == XR_REC_RETENTION && n_chunks > 1 && scratch && chunk_len % REC_TOKENS == 0),
-               "recurrence: chunks are for retention, with room for their states");
+    XR_REQUIRE(!chunks || (mode != XR_REC_DELTA && n_chunks > 1 && scratch && chunk_len % REC_TOKENS == 0),
+               "recurrence: chunks are for retention and wkv, with room for their states");
+    XR_REQUIRE(!chunks || mode != XR_REC_WKV || prod, "recurrence: wkv in chunks needs room for the chunks' decay products");
     XR_REQUIRE(!chunks || (long long)B * n_chunks <= 65535, "recurrence: %d requests of %d chunks", B, n_chunks);
-    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, chunks ? 1 : 0, chunk_len, n_chunks, scratch, act};
+    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, chunks ? 1 : 0, chunk_len, n_chunks, scratch, act, prod};
     const int R = rec_lanes(D), cols = 256 / R, per = (D + R - 1) / R;
     dim3 grid((Dv + cols - 1) / cols, H, chunks ? B * n_chunks : B);
 #define REC(M)                                                                          \
@@ -357,9 +385,12 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
     else REC(XR_REC_RETENTION);
     if (chunks) {
         const int per_head = per * Dv * R;
-        k_retention_carry<<<dim3((per_head + 255) / 256, H, B), 256, 0, stream>>>(a, per_head);
+        const dim3 cgrid((per_head + 255) / 256, H, B);
+        if (mode == XR_REC_WKV) k_retention_carry<true><<<cgrid, 256, 0, stream>>>(a, per_head, R);
+        else k_retention_carry<false><<<cgrid, 256, 0, stream>>>(a, per_head, R);
         a.pass = 2;
-        REC(XR_REC_RETENTION);
+        if (mode == XR_REC_WKV) REC(XR_REC_WKV);
+        else REC(XR_REC_RETENTION);
     }
 #undef REC
     XR_CHECK_LAUNCH("linear_recurrence");

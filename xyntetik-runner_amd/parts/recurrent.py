@@ -233,6 +233,8 @@ class TimeMixWKV(Mixer):
     def param_specs(self) -> Dict[str, ParamSpec]:
         E, N, n = self.hidden_size, self.size, self.names
         rank = max(4, E // 10)      # what the random-weights mode writes; a file may bring any
+        if rank >= 64:
+            rank = rank // 64 * 64
         specs = {n["mu"] + s: ParamSpec((E,), role="vector", init="around:0.5:0.25") for s in self.MIXES}
         for key in ("r", "k", "v", "g"):
             specs[n[key]] = ParamSpec((N, E))
@@ -251,9 +253,14 @@ class TimeMixWKV(Mixer):
         w1, w2 = tensors[n["w1"]], tensors[n["w2"]]
         if w1.shape[0] != w2.shape[1]:
             raise ValueError(f"wkv time mixing: the decay's matrices {tuple(w1.shape)} and {tuple(w2.shape)} do not meet")
-        self.decay_rank = int(w1.shape[0])
+        self.decay_rank = rank = int(w1.shape[0])
         self.mu = torch.stack([tensors[n["mu"] + s].float() for s in self.MIXES]).contiguous()
-        self.w_rkvg = torch.stack([tensors[n[key]] for key in ("r", "k", "v", "g")]).contiguous()      # [4, N, E]: one launch
+        # r, k, v and the gate read a mix each: four products of the full width, each by the kernel a projection gets
+        self.w_rkvg = [rt.ops.pack_weight(tensors[n[key]].contiguous()) for key in ("r", "k", "v", "g")]
+        if rank % 8:        # the inner side in whole groups of 8 (what the matrix cores take): rows and columns of
+            pad = 8 - rank % 8      # zeros, whose tanh is zero and adds nothing
+            w1 = torch.cat([w1, w1.new_zeros((pad, w1.shape[1]))], dim=0)
+            w2 = torch.cat([w2, w2.new_zeros((w2.shape[0], pad))], dim=1)
         self.w1, self.w2 = rt.ops.pack_weight(w1.contiguous()), rt.ops.pack_weight(w2.contiguous())
         self.w0 = tensors[n["w0"]].float().contiguous()
         self.u = tensors[n["u"]].float().contiguous()
@@ -268,7 +275,8 @@ class TimeMixWKV(Mixer):
         T = h.shape[0]
         mixes = ops.token_shift(h, self.mu, cache.states["mixer.shift"], ctx, dt)          # [T, 5 E]: r, k, v, g, w
         proj = torch.empty((T, 4 * N), dtype=torch.float32, device=h.device)
-        ops.heads_linear(mixes, self.w_rkvg, proj, 4, E, N)
+        for s, w in enumerate(self.w_rkvg):
+            ops.linear(mixes[:, s * E:(s + 1) * E], w, out=proj[:, s * N:(s + 1) * N])
         r, k, v, gate = proj[:, :N], proj[:, N:2 * N], proj[:, 2 * N:3 * N], proj[:, 3 * N:]
         inner = ops.linear(mixes[:, 4 * E:], self.w1, out_dtype=torch.float32)
         ops.act_rows_(inner, "tanh")
