@@ -108,8 +108,19 @@ TINY_D6 = {
 
 # (configuration, seed, deviation of the matrices: smaller where a factor above one and two passes over the
 # whole model would otherwise make single rows pass a rounding on a hundredfold, in 32 bits as in 16)
+# a width that is a multiple of nothing the kernels like (no 16-byte rows, no matrix cores), every head count odd
+TINY_D7 = {
+    "architecture": "Dinasun", "vocab": 61, "width": 30, "norm": {"eps": 1e-5}, "residual_mult": 0.75,
+    "embedding": {"scale": 1.3},
+    "loop": {"start": 1, "stop": 2, "times": 2},
+    "layers": [
+        with_ff(wkv(3, 6), moe(10, 3, 2, shared=7)),
+        with_ff(attention(3, 3, 10, 0.3, coef=0.2, every=7), moe(9, 2, 2)),
+    ],
+}
+
 CONFIGS = {"D1": (TINY_D1, 31, 0.2), "D2": (TINY_D2, 32, 0.2), "D3": (TINY_D3, 33, 0.1), "D4": (TINY_D4, 34, 0.2),
-           "D5": (TINY_D5, 35, 0.2), "D6": (TINY_D6, 36, 0.2)}
+           "D5": (TINY_D5, 35, 0.2), "D6": (TINY_D6, 36, 0.2), "D7": (TINY_D7, 37, 0.2)}
 
 
 def make_model(which: str, folder: str, std: float = 0.0) -> str:

@@ -2,7 +2,7 @@
 whole prompts, prompts with their last tokens one by one, portions down to two tokens, mixed
 batches in pools so small that pages and state slots are used again, long decoding through
 recorded steps, and greedy generation through the engine's own entry point and scheduler.
-Six configurations that differ in every size and constant (``dinasun_tiny``)."""
+Seven configurations that differ in every size and constant (``dinasun_tiny``)."""
 import io
 import json
 import os
@@ -33,6 +33,7 @@ WORKLOAD = {
     "D4": ([2, 65, 99, 330], 80),           # position 99 is the first with the higher temperature: as the last of a prompt, and decoded
     "D5": ([1, 30, 90], 50),
     "D6": ([1, 2, 17, 40], 12),
+    "D7": ([2, 33, 70], 20),
 }
 
 
@@ -96,7 +97,8 @@ def steps_for(schedule, reqs, plens, extra):
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which,page_size", [("D1", 16), ("D2", 8), ("D3", 64), ("D4", 64), ("D5", 32), ("D6", 4)])
+@pytest.mark.parametrize("which,page_size", [("D1", 16), ("D2", 8), ("D3", 64), ("D4", 64), ("D5", 32), ("D6", 4),
+                                              ("D7", 16)])
 def test_every_way_of_cutting_gives_the_plain_logits(models, tmp_path, which, page_size, dtype, schedule):
     d, cfg, w, reqs, plens, want = models[which]
     steps = steps_for(schedule, reqs, plens, WORKLOAD[which][1])
@@ -143,6 +145,21 @@ def test_long_decoding_through_recorded_steps(models, tmp_path, dtype, which):
     out, runner = run_replay(d, dtype, steps, tmp_path, 16)
     assert runner.graphs.replays >= 290
     check(traces.collect(steps, out, cfg["vocab"]), {"long": wanted}, dtype, "long decoding")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_long_prompt_whole_and_in_portions(models, tmp_path, dtype):
+    """1,300 tokens in one step (time mixing then runs its rows as chunks side by side, attention in whole
+    tiles), the same in two long portions around a short one, and 20 more one by one behind either."""
+    d, cfg, w, *_ = models["D1"]
+    toks = prompt_ids(1320, cfg["vocab"], 78)
+    wanted = {"long": P.forward(cfg, w, toks)}
+    whole = traces.tail_one_by_one({"long": toks}, tail=20)
+    out, _ = run_replay(d, dtype, whole, tmp_path / "w", 64)
+    check(traces.collect(whole, out, cfg["vocab"]), wanted, dtype, "long prompt")
+    cut = traces.portions({"long": toks}, sizes=(1100, 2, 198, 1, 1, 18))
+    out, _ = run_replay(d, dtype, cut, tmp_path / "c", 16)
+    check(traces.collect(cut, out, cfg["vocab"]), wanted, dtype, "long prompt in portions")
 
 
 def test_eager_and_recorded_steps_agree(models, tmp_path):
