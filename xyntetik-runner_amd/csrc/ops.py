@@ -71,7 +71,7 @@ _PROTOS = {
     "xr_polynorm": [_p, _p, _p, _i, _i, _i, _f, _i, _i, _p],
     "xr_rotate_rows": [_p, _p, _p, _i, _i, _i, _i, _i, _f, _p],
     "xr_gated_rmsnorm": [_p, _p, _p, _p, _i, _i, _i, _i, _f, _i, _i, _i, _p],
-    "xr_act_rows": [_p, _i, _i, _i, _i, _p],
+    "xr_act_rows": [_p, _i, _i, _i, _i, _p, _i, _p],
     "xr_embedding_pairs": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _p],
     "xr_streams_expand": [_p, _p, _i, _i, _i, _p],
     "xr_streams_sum": [_p, _p, _i, _i, _i, _p],
@@ -841,12 +841,22 @@ class Ops:
 
     def act_rows_(self, x: torch.Tensor, activation: str = "silu") -> None:
         """``x <- act(x)`` in place on a 32-bit view ``[rows, width]`` with unit column stride."""
+        self._act_rows(x, activation, None)
+
+    def act_rows(self, x: torch.Tensor, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
+        """``act(x)`` of a 32-bit view ``[rows, width]`` as contiguous rows in ``out_dtype`` (what a product reads next)."""
+        out = torch.empty(tuple(x.shape), dtype=out_dtype, device=x.device)
+        self._act_rows(x, activation, out)
+        return out
+
+    def _act_rows(self, x, activation, out) -> None:
         self._dev(x)
         if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1:
-            raise KernelError("act_rows_: x must be a float32 view [rows, width] with unit column stride")
+            raise KernelError("act_rows: x must be a float32 view [rows, width] with unit column stride")
         if activation not in ROW_ACTIVATIONS:
-            raise KernelError(f"act_rows_: activation {activation!r} is not built ({', '.join(sorted(ROW_ACTIVATIONS))})")
-        self.lib.check(self.lib.xr_act_rows(x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), ROW_ACTIVATIONS[activation], _stream()))
+            raise KernelError(f"act_rows: activation {activation!r} is not built ({', '.join(sorted(ROW_ACTIVATIONS))})")
+        self.lib.check(self.lib.xr_act_rows(x.data_ptr(), x.shape[0], x.shape[1], x.stride(0), ROW_ACTIVATIONS[activation],
+                                            _ptr(out), dtype_code(out.dtype) if out is not None else XR_F32, _stream()))
 
     # -- an embedding with a hashed table of token pairs --------------------------
     def embedding_pairs(self, table: torch.Tensor, pairs: Optional[torch.Tensor], norm_w: Optional[torch.Tensor], ids, ctx,

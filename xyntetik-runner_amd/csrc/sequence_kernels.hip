@@ -451,24 +451,31 @@ extern "C" int xr_gated_rmsnorm(void* out, const float* o, const float* gate, co
     return XR_OK;
 }
 
-// ---------------------------------------------------------------- an activation on 32-bit rows, in place
-// x[t][c] <- act(x[t][c]) for the first W columns of rows of stride ld; act 1 = SiLU, 2 = tanh.
+// ---------------------------------------------------------------- an activation on 32-bit rows
+// x[t][c] <- act(x[t][c]) for the first W columns of rows of stride ld, in place; or, with `out`, into
+// contiguous rows [T, W] of the type the next product reads.  act 1 = SiLU, 2 = tanh.
 #define XR_ACT_ROWS_TANH 2
-__global__ void k_act_rows(float* __restrict__ x, int W, int ld, size_t n, int act) {
+template <typename TO>
+__global__ void k_act_rows(float* __restrict__ x, TO* __restrict__ out, int W, int ld, size_t n, int act) {
     const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= n) return;
     const size_t t = i / W;
     float* p = x + t * ld + (i - t * W);
     const float v = *p;
-    *p = act == XR_ACT_ROWS_TANH ? tanhf(v) : v / (1.0f + expf(-v));
+    const float y = act == XR_ACT_ROWS_TANH ? tanhf(v) : v / (1.0f + expf(-v));
+    if (out) st<TO>(out, i, y);
+    else *p = y;
 }
 
-extern "C" int xr_act_rows(float* x, int T, int W, int ld, int act, hipStream_t stream) {
+extern "C" int xr_act_rows(float* x, int T, int W, int ld, int act, void* out, int out_dtype, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && W > 0 && ld >= W, "act_rows: bad sizes T=%d W=%d ld=%d", T, W, ld);
     XR_REQUIRE(act == XR_CONV_SILU || act == XR_ACT_ROWS_TANH, "act_rows: activation %d is not built (1 = SiLU, 2 = tanh)", act);
+    XR_REQUIRE(!out || out_dtype == XR_F32 || out_dtype == XR_BF16, "act_rows: output type %d", out_dtype);
     const size_t n = (size_t)T * W;
     if (n == 0) return XR_OK;
-    k_act_rows<<<(unsigned)((n + 255) / 256), 256, 0, stream>>>(x, W, ld, n, act);
+    const unsigned blocks = (unsigned)((n + 255) / 256);
+    if (out && out_dtype == XR_BF16) k_act_rows<bf16_t><<<blocks, 256, 0, stream>>>(x, (bf16_t*)out, W, ld, n, act);
+    else k_act_rows<float><<<blocks, 256, 0, stream>>>(x, (float*)out, W, ld, n, act);
     XR_CHECK_LAUNCH("act_rows");
     return XR_OK;
 }

@@ -279,8 +279,7 @@ class TimeMixWKV(Mixer):
             ops.linear(mixes[:, s * E:(s + 1) * E], w, out=proj[:, s * N:(s + 1) * N])
         r, k, v, gate = proj[:, :N], proj[:, N:2 * N], proj[:, 2 * N:3 * N], proj[:, 3 * N:]
         inner = ops.linear(mixes[:, 4 * E:], self.w1, out_dtype=torch.float32)
-        ops.act_rows_(inner, "tanh")
-        x = ops.linear(inner if self.rt.is_fp32 else ops.convert(inner, dt), self.w2, bias=self.w0, out_dtype=torch.float32)
+        x = ops.linear(ops.act_rows(inner, "tanh", dt), self.w2, bias=self.w0, out_dtype=torch.float32)
         o = ops.linear_recurrence("wkv", r, k, v, cache.states["mixer.S"], ctx, H, H, D, D, gate=x, decay=self.u)
         return ops.gated_rmsnorm(o, gate, self.w_norm, H, D, self.eps, dt)
 
