@@ -340,7 +340,7 @@ def dinasun_config(width, layers, vocab=32000):
     wkv = {"type": "wkv", "mixer": {"heads": width // 64, "dim": 64}, "mlp": moe}
     att = {"type": "attention", "mixer": {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
                                           "q_temp": {"coef": 0.1, "every": 1024}}, "mlp": moe}
-    cfg = {"architecture": "Dinasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.7,
+    cfg = {"architecture": "Dinasun", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "residual_mult": 0.8,
            "embedding": {"scale": 1.0}, "layers": [wkv if i % 2 == 0 else att for i in range(distinct)]}
     if again:
         start = (distinct - again) // 2
