@@ -405,6 +405,73 @@ def test_gated_experts_chosen_by_token_id(ops, n, top, E, F, T, dt, tol):
     close(base.cpu().numpy(), want + 1.0, tol, "experts added to what is there")
 
 
+# ----------------------------------------------------------------------------- a one-layer model with made weights
+def needle_model():
+    """One attention layer, two heads on one key head, no feed-forward.  Token 1 (the needle) has a key along
+    channel 0, where every query lies (through the query's bias, whatever the token), with a score of 36 before the
+    bias of the distance; token 0 (the filler) has a key along channel 1, with a score around 0.  The value is the
+    key as projected, so the needle's lands in channel 0 of a head's output; the output matrix brings head 0's
+    there to stream channel 5 and head 1's to channel 4, which rows 3 and 2 of the embedding read as logits."""
+    E, V, H, D = 8, 4, 2, 4
+    rng = np.random.default_rng(4)
+    cfg = {"architecture": "Dinasun", "vocab": V, "width": E, "norm": {"eps": 1e-6}, "residual_mult": 1.0,
+           "layers": [{"type": "attention", "mixer": {"heads": H, "kv_heads": 1, "dim": D, "vdim": D, "scale": 1.0}, "mlp": None}]}
+    emb = np.zeros((V, E)); emb[0, 1] = 1.0; emb[1, 0] = 1.0; emb[2, 4] = 1.0; emb[3, 5] = 1.0
+    w = {"embed": emb}
+    for n in ("l0.norm1", "l0.norm1b", "final.norm"):
+        w[n], w[n + ".b"], w[n + ".alpha"] = np.ones(E), np.zeros(E), np.asarray(1.0)
+    wq = rng.normal(size=(H * D, E)) * 0.01
+    bq = np.zeros(H * D); bq[0] = bq[D] = 1.0                        # channel 0 of both heads
+    wk = rng.normal(size=(D, E)) * 0.01
+    wk[0, 0] = 1.0                                                    # the needle's key: channel 0
+    wk[1, 1] = 1.0                                                    # a filler's: channel 1
+    qn, kn = np.ones(D), np.ones(D)
+    qn[0] = kn[0] = 3.0                                               # a unit vector of 4 channels has 2 in its one channel: 6 x 6
+    o = rng.normal(size=(E, H * D)) * 0.01
+    o[5, 0] = 2.0
+    o[4, D] = 2.0
+    w.update({"l0.mix.q": wq, "l0.mix.q.b": bq, "l0.mix.k": wk, "l0.mix.k.b": np.zeros(D), "l0.mix.q.norm": qn, "l0.mix.k.norm": kn,
+              "l0.mix.o": o})
+    return cfg, w
+
+
+def engine_logits(cfg, w, steps, dtype, page, max_tokens, tmp_path):
+    from xyntetik_runner_amd.config import config_from_dict
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    arch, typed = config_from_dict(cfg)
+    tensors = {k: torch.tensor(v, dtype=torch.float32) for k, v in w.items()}
+    runner = ModelRunner(arch.build_spec(typed), tensors, dtype, max_tokens=max_tokens, page_size=page, max_requests=2)
+    for lc in runner.storage.layers:
+        if lc.owns and lc.k is not None:
+            lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+    out = str(tmp_path / "out")
+    replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+    return traces.collect(steps, out, cfg["vocab"])
+
+
+@pytest.mark.parametrize("page", [16, 64])
+@pytest.mark.parametrize("decode_from", [None, 30])
+def test_one_key_that_stands_out_through_the_engine(tmp_path, page, decode_from):
+    """The needle at the start, at a page's last and first place: 1,500 (decoded: 800) tokens later, among the fillers, the
+    head of slope 1/256 still reads it (logit 2), the head of slope 1/16 has lost it since some 500 tokens
+    (logit 3) and had it before.  In a prompt's portions and with all but 30 positions decoded one by one."""
+    cfg, w = needle_model()
+    n = 1560 if decode_from is None else 900
+    for jstar in (3, 63, 64):
+        toks = [0] * n
+        toks[jstar] = 1
+        want = P.forward(cfg, w, toks)
+        assert want[-1, 2] > 0.5 and want[-1, 3] < 0.05 and want[jstar + 100, 3] > 0.5, "the made weights do not show the needle"
+        assert want[jstar - 1, 2] < 0.05, "the needle shows before it is there"
+        if decode_from is None:
+            steps = traces.portions({"a": toks}, sizes=(17, 2, 40, 3, 1100, 64))
+        else:
+            steps = traces.tail_one_by_one({"a": toks}, tail=n - decode_from)
+        got = engine_logits(cfg, w, steps, "float32", page, -(-n // 64) * 64 + 64, tmp_path / f"{jstar}")
+        close(got["a"], want, 1e-5, f"needle at {jstar}")
+
+
 # ----------------------------------------------------------------------------- whole models at a sequence's start
 def test_first_tokens_of_a_sequence(tmp_path):
     """Sequences of one, two and three tokens beside a longer one in a mixed batch: the row before the
