@@ -52,6 +52,11 @@ def first_needed_position(n_tokens: int, window: Optional[int]) -> int:
     return max(0, n_tokens - window + 1)
 
 
+def kept_pages(spec: KVSpec, page_size: int) -> int:
+    """The pages at a request's start that a windowed group never gives back (``KVSpec.keep_first``)."""
+    return -(-spec.keep_first // page_size) if (spec.window is not None and spec.keep_first > 0) else 0
+
+
 def pages_for_spec(spec: KVSpec, page_size: int, max_tokens: int, max_requests: int,
                    max_step_tokens: Optional[int] = None) -> int:
     """How many pages a group needs so that ``max_requests`` requests holding ``max_tokens`` tokens
@@ -69,7 +74,7 @@ def pages_for_spec(spec: KVSpec, page_size: int, max_tokens: int, max_requests: 
         return -(-full // spec.stride) + max_requests
     if spec.window is None or max_step_tokens is None:
         return full
-    per_request = -(-spec.window // page_size) + 2
+    per_request = -(-spec.window // page_size) + 2 + kept_pages(spec, page_size)
     return min(full, max_requests * per_request + -(-int(max_step_tokens) // page_size))
 
 
@@ -114,7 +119,7 @@ class CacheManager:
         best = 1 << 62
         for g in self.groups:
             if g.spec.window is not None:
-                behind = -(-g.spec.window // self.page_size) + 1
+                behind = -(-g.spec.window // self.page_size) + 1 + kept_pages(g.spec, self.page_size)
                 best = min(best, max(1, (g.pool.size - behind) * self.page_size))
         return best
 
@@ -152,7 +157,8 @@ class CacheManager:
             want = self.pages_for(new_len, gi)
             # pages wholly below the window of the first new query are never read or written
             lo_page = first_needed_position(rc.n_tokens, g.spec.window) // self.page_size
-            need.append(sum(1 for i in range(have, want) if i >= lo_page))
+            kept = kept_pages(g.spec, self.page_size)
+            need.append(sum(1 for i in range(have, want) if i >= lo_page or i < kept))
         return need
 
     def can_reserve(self, req_id: Hashable, new_len: int, spare: Optional[List[int]] = None) -> bool:
@@ -200,8 +206,9 @@ class CacheManager:
         for gi, g in enumerate(self.groups):
             table = rc.tables[gi]
             lo_page = first_needed_position(rc.n_tokens, g.spec.window) // self.page_size
+            kept = kept_pages(g.spec, self.page_size)
             for i in range(len(table), self.pages_for(new_len, gi)):
-                table.append(g.pool.take() if i >= lo_page else -1)
+                table.append(g.pool.take() if (i >= lo_page or i < kept) else -1)
 
     def advance(self, req_id: Hashable, new_len: int) -> None:
         """Positions below ``new_len`` are now cached; give back pages a window has passed."""
@@ -214,7 +221,7 @@ class CacheManager:
             g = self.groups[gi]
             lo_page = first_needed_position(new_len, g.spec.window) // self.page_size
             table = rc.tables[gi]
-            for i in range(min(lo_page, len(table))):
+            for i in range(kept_pages(g.spec, self.page_size), min(lo_page, len(table))):
                 if table[i] >= 0:
                     g.pool.give(table[i])
                     table[i] = -1
@@ -253,6 +260,7 @@ class CacheManager:
         for rc in self.requests.values():
             for gi, g in enumerate(self.groups):
                 lo = first_needed_position(rc.n_tokens, g.spec.window)
-                for pos in range(lo, rc.n_tokens // g.spec.stride):
+                kept = min(g.spec.keep_first, rc.n_tokens) if g.spec.window is not None else 0
+                for pos in list(range(min(kept, lo))) + list(range(lo, rc.n_tokens // g.spec.stride)):
                     if rc.tables[gi][pos // self.page_size] < 0:
                         raise AssertionError(f"request {rc.req_id!r}: position {pos} of group {gi} has no page")

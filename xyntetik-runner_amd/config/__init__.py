@@ -3,12 +3,13 @@ from .llama import LlamaConfig, RopeScaling
 from .suripel import SuripelConfig
 from .sugosun import SugosunConfig
 from .dinasun import DinasunConfig
+from .kegorax import KegoraxConfig
 from .spec import PartSpec, LayerSpec, ExecStep, ModelSpec
 from .registry import (register_architecture, unregister_architecture, get_architecture,
                        known_architectures, load_config, config_from_dict, Architecture)
 
 __all__ = [
-    "ConfigError", "Fields", "read_config_json", "architecture_name", "LlamaConfig", "RopeScaling", "SuripelConfig", "SugosunConfig", "DinasunConfig",
+    "ConfigError", "Fields", "read_config_json", "architecture_name", "LlamaConfig", "RopeScaling", "SuripelConfig", "SugosunConfig", "DinasunConfig", "KegoraxConfig",
     "PartSpec", "LayerSpec", "ExecStep", "ModelSpec", "register_architecture",
     "unregister_architecture", "get_architecture", "known_architectures", "load_config",
     "config_from_dict", "Architecture",

@@ -55,11 +55,12 @@ class ExecStep:
     ``cache_of`` is the index of an earlier entry whose cache this entry reads
     instead of owning one; such an entry writes no keys or values.
     ``enters``: the model's ``injection`` runs right before this entry (the first layer of a pass
-    over a looped span, say).
+    over a looped span, say); ``pass_index`` tells it which pass that is, counted from 0.
     """
     layer: int
     cache_of: Optional[int] = None
     enters: bool = False
+    pass_index: int = 0
 
 
 @dataclass(frozen=True)

@@ -63,7 +63,8 @@ struct AttnArgs {
     float* part_ml;         // [slots, Hk, ROWS, 2]
     int n_items, n_cta_items, H, Hk, page_shift, page_mask, page_size;
     float scale;
-    int window;
+    int window;             // > 0: a row at position p reads the keys from p - window + 1 on
+    int chunk;              // > 0: it reads from p - p mod chunk on (its own chunk of positions, counted from 0)
     const float* slopes;    // [H], or null: slopes[h] * (i - j) is taken off the score of query i and key j
 };
 
@@ -489,7 +490,7 @@ __global__ __launch_bounds__(CtaShape::THREADS, 1) void k_attn_cta(AttnArgs a) {
         const bool row_ok = tok < q_len;
         w.row_ok = row_ok;
         w.pos = start + tok;
-        w.lo = (a.window > 0 && w.pos - a.window + 1 > 0) ? w.pos - a.window + 1 : 0;
+        w.lo = a.chunk > 0 ? w.pos - w.pos % a.chunk : (a.window > 0 && w.pos - a.window + 1 > 0) ? w.pos - a.window + 1 : 0;
         w.lg = lg;
         w.sb = SLOPES ? a.slopes[kvh * G + hg] / a.scale : 0.f;
         const bf16_t* qp = a.q + ((size_t)(row_ok ? it[5] + tok : it[5]) * a.H + kvh * G + hg) * HD + lg * 8;
@@ -785,7 +786,7 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
     const bool row_ok = tok < q_len;
     const int t = q0 + tok, h = kvh * G + hg;
     const int pos = start + tok;
-    const int lo = (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
+    const int lo = a.chunk > 0 ? pos - pos % a.chunk : (a.window > 0 && pos - a.window + 1 > 0) ? pos - a.window + 1 : 0;
     const float sb = SLOPES ? a.slopes[h] / a.scale : 0.f;
 
     bf16x8 qf[KD];
@@ -1067,12 +1068,12 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
                                  const int* cu_q,
                                  const int* starts, const int* block_table, int table_stride, float* part_o,
                                  float* part_ml, int H, int Hk, int D, int page_size, float scale, int window,
-                                 const float* slopes, hipStream_t stream) {
+                                 int chunk, const float* slopes, hipStream_t stream) {
     XR_REQUIRE(D == HD, "attention: this library is compiled for head size %d, got %d", HD, D);
     XR_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
     int shift = ilog2_exact(page_size);
     XR_REQUIRE(shift >= 4, "attention: the MFMA kernel needs a page size that is a power of two of at least 16, got %d", page_size);
-    XR_REQUIRE(window >= 0, "attention: window %d is negative", window);
+    XR_REQUIRE(window >= 0 && chunk >= 0, "attention: window %d or chunk %d is negative", window, chunk);
     XR_REQUIRE(n_items >= 0 && n_jobs >= 0 && n_cta_items >= 0, "attention: negative work counts");
     XR_REQUIRE((long long)n_cta_items * Hk < (1LL << 31) && (long long)n_items * Hk < (1LL << 31), "attention: %d items of %d key/value heads are more workgroups than a launch takes", n_items + n_cta_items, Hk);
     XR_REQUIRE(n_cta_items == 0 || page_size >= 32, "attention: 128-row items need pages of at least 32 positions, got %d", page_size);
@@ -1083,7 +1084,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     // the list begins with the items of the workgroup kernel
     a.cta_items = items; a.n_cta_items = n_cta_items; a.items = items + (size_t)n_cta_items * ITEM_INTS; a.cu_q = cu_q; a.starts = starts; a.block_table = block_table; a.table_stride = table_stride;
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
-    a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window;
+    a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window; a.chunk = chunk;
     a.slopes = slopes;
     XR_REQUIRE(!slopes || scale > 0.f, "attention: distance slopes need a positive scale, got %g", (double)scale);
     if (n_cta_items > 0) {

@@ -10,6 +10,10 @@
 // softmax runs over blocks of 64 keys with a running maximum and sum, which gives the
 // same value up to rounding.  With `slopes` (one number a query head) a bias that grows with the distance is
 // taken off every score: s_t = (q . K_t) * scale - slope_h * (p - t).
+// Other masks: `chunk` > 0: lo = p - p mod chunk (a position reads its own chunk of positions, counted from 0);
+// `keep` > 0: the keys [0, keep) are read as well wherever lo lies.  `sinks` (one number a query head): the
+// softmax's denominator also holds exp(sink_h), an entry that has no key and no value.  Values may have another
+// size than keys (Dv; cache layout K [page][kv_head][slot][D], V [page][kv_head][Dv][slot]).
 #include "common.h"
 
 #define AR_MAX_D 256
@@ -18,14 +22,16 @@ template <typename T>
 __global__ __launch_bounds__(64) void k_attention_ref(
     T* __restrict__ out, const T* __restrict__ q, const T* __restrict__ kc, const T* __restrict__ vc,
     const int* __restrict__ positions, const int* __restrict__ req_of_token,
-    const int* __restrict__ block_table, int table_stride, int H, int Hk, int D, int page_shift,
-    int page_mask, int page_size, float scale, int window, const float* __restrict__ slopes) {
+    const int* __restrict__ block_table, int table_stride, int H, int Hk, int D, int Dv, int page_shift,
+    int page_mask, int page_size, float scale, int window, int chunk, int keep, const float* __restrict__ slopes,
+    const float* __restrict__ sinks) {
     __shared__ float qs[AR_MAX_D];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[t];
     const int req = req_of_token[t];
     const int kvh = h / (H / Hk);
-    const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int lo = chunk > 0 ? pos - pos % chunk : (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int kept = keep < lo ? keep : lo;         // kept keys [0, kept) lie below the row's own range
     const T* qrow = q + ((size_t)t * H + h) * D;
     for (int d = lane; d < D; d += 64) qs[d] = ld<T>(qrow, d);
     __syncthreads();
@@ -37,9 +43,10 @@ __global__ __launch_bounds__(64) void k_attention_ref(
 #pragma unroll
     for (int dd = 0; dd < AR_MAX_D / 64; ++dd) acc[dd] = 0.f;
 
-    for (int k0 = lo; k0 <= pos; k0 += 64) {
+    for (int seg = kept > 0 ? 0 : 1; seg < 2; ++seg)
+    for (int k0 = seg ? lo : 0, last = seg ? pos : kept - 1; k0 <= last; k0 += 64) {
         const int key = k0 + lane;
-        const bool valid = key <= pos;
+        const bool valid = key <= last;
         float s = -INFINITY;
         if (valid) {
             const int page = bt[key >> page_shift];
@@ -51,40 +58,50 @@ __global__ __launch_bounds__(64) void k_attention_ref(
         }
         const float mn = fmaxf(m, wave_max(s));
         const float p = valid ? expf(s - mn) : 0.f;
-        const float corr = expf(m - mn);
+        const float corr = m == -INFINITY ? 0.f : expf(m - mn);
         l = l * corr + wave_sum(p);
 #pragma unroll
         for (int dd = 0; dd < AR_MAX_D / 64; ++dd) acc[dd] *= corr;
-        const int nk = (pos - k0 + 1) < 64 ? (pos - k0 + 1) : 64;
+        const int nk = (last - k0 + 1) < 64 ? (last - k0 + 1) : 64;
         for (int j = 0; j < nk; ++j) {
             const float pj = __shfl(p, j, 64);
             const int kj = k0 + j;
             const int page = bt[kj >> page_shift];
             const int off = kj & page_mask;
-            const T* vb = vc + ((size_t)page * Hk + kvh) * D * page_size + off;
+            const T* vb = vc + ((size_t)page * Hk + kvh) * Dv * page_size + off;
 #pragma unroll
             for (int dd = 0; dd < AR_MAX_D / 64; ++dd) {
                 const int d = lane + 64 * dd;
-                if (d < D) acc[dd] = fmaf(pj, ld<T>(vb, (size_t)d * page_size), acc[dd]);
+                if (d < Dv) acc[dd] = fmaf(pj, ld<T>(vb, (size_t)d * page_size), acc[dd]);
             }
         }
         m = mn;
     }
-    T* orow = out + ((size_t)t * H + h) * D;
+    if (sinks) {            // one more entry of the denominator, with nothing to add to the output
+        const float sk = sinks[h];
+        const float mn = fmaxf(m, sk);
+        const float corr = expf(m - mn);
+        l = l * corr + expf(sk - mn);
+#pragma unroll
+        for (int dd = 0; dd < AR_MAX_D / 64; ++dd) acc[dd] *= corr;
+    }
+    T* orow = out + ((size_t)t * H + h) * Dv;
 #pragma unroll
     for (int dd = 0; dd < AR_MAX_D / 64; ++dd) {
         const int d = lane + 64 * dd;
-        if (d < D) st<T>(orow, d, acc[dd] / l);
+        if (d < Dv) st<T>(orow, d, acc[dd] / l);
     }
 }
 
 extern "C" int xr_attention_ref(void* out, const void* q, const void* k_cache, const void* v_cache,
                                 const int* positions, const int* req_of_token, const int* block_table,
-                                int table_stride, int T, int H, int Hk, int D, int page_size, float scale,
-                                int window, int dtype, const float* slopes, hipStream_t stream) {
+                                int table_stride, int T, int H, int Hk, int D, int Dv, int page_size, float scale,
+                                int window, int chunk, int keep, int dtype, const float* slopes, const float* sinks,
+                                hipStream_t stream) {
     XR_REQUIRE(T >= 0 && H > 0 && Hk > 0 && D > 0, "attention: bad sizes T=%d H=%d Hk=%d D=%d", T, H, Hk, D);
     XR_REQUIRE(H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
-    XR_REQUIRE(D <= AR_MAX_D, "attention: head size %d exceeds %d", D, AR_MAX_D);
+    XR_REQUIRE(D <= AR_MAX_D && Dv > 0 && Dv <= AR_MAX_D, "attention: head size %d or value size %d exceeds %d", D, Dv, AR_MAX_D);
+    XR_REQUIRE(chunk >= 0 && keep >= 0, "attention: chunk %d or kept keys %d are negative", chunk, keep);
     int shift = ilog2_exact(page_size);
     XR_REQUIRE(shift >= 0, "attention: page size %d is not a power of two", page_size);
     XR_REQUIRE(window >= 0, "attention: window %d is negative", window);
@@ -93,11 +110,11 @@ extern "C" int xr_attention_ref(void* out, const void* q, const void* k_cache, c
     if (dtype == XR_F32)
         k_attention_ref<float><<<grid, 64, 0, stream>>>((float*)out, (const float*)q, (const float*)k_cache,
                                                         (const float*)v_cache, positions, req_of_token, block_table,
-                                                        table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window, slopes);
+                                                        table_stride, H, Hk, D, Dv, shift, page_size - 1, page_size, scale, window, chunk, keep, slopes, sinks);
     else if (dtype == XR_BF16)
         k_attention_ref<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)out, (const bf16_t*)q, (const bf16_t*)k_cache,
                                                          (const bf16_t*)v_cache, positions, req_of_token, block_table,
-                                                         table_stride, H, Hk, D, shift, page_size - 1, page_size, scale, window, slopes);
+                                                         table_stride, H, Hk, D, Dv, shift, page_size - 1, page_size, scale, window, chunk, keep, slopes, sinks);
     else { xr_set_error("attention: bad dtype %d", dtype); return XR_BAD_ARG; }
     XR_CHECK_LAUNCH("attention_ref");
     return XR_OK;

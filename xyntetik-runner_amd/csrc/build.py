@@ -36,7 +36,7 @@ UNITS: Dict[str, dict] = {
     "kernels": {
         "sources": ["errors.hip", "basic_kernels.hip", "gemm_ref.hip", "attention_ref.hip",
                     "sampling.hip", "gemm_mfma.hip", "sequence_kernels.hip", "recurrent_kernels.hip",
-                    "attention_pooled.hip", "stream_kernels.hip", "latent_kernels.hip", "moe_kernels.hip", "grouped_mfma.hip"],
+                    "attention_pooled.hip", "stream_kernels.hip", "latent_kernels.hip", "moe_kernels.hip", "grouped_mfma.hip", "mixer_kernels.hip"],
         "defines": [],
     },
 }

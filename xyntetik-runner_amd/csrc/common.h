@@ -80,11 +80,18 @@ __host__ __device__ inline uint32_t pack_bf16x2(float lo, float hi) {
 // gate (the products' epilogues and k_gate_mul) takes the code as an argument.
 #define XR_ACT_SILU 0
 #define XR_ACT_CLAMPED_SWISH 1      // takes a number (the limit) and shapes both branches: see gate_value below
-#define XR_ACT_COUNT 2
+#define XR_ACT_GELU_TANH 2          // 0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))
+#define XR_ACT_COUNT 3
 #if defined(__HIP_DEVICE_COMPILE__)
 // FAST: with the hardware's 2^x and reciprocal (1 ulp each)
 template <bool FAST> __device__ inline float gate_act(int act, float g) {
     switch (act) {
+    case XR_ACT_GELU_TANH: {
+        // 0.5 g (1 + tanh(y)) = g / (1 + exp(-2 y)), y = sqrt(2/pi) (g + 0.044715 g^3)
+        const float y2 = 1.5957691216f * fmaf(0.044715f * g * g, g, g);
+        return FAST ? g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(y2 * -1.44269504f))
+                    : g / (1.0f + expf(-y2));
+    }
     default:    // XR_ACT_SILU: g / (1 + exp(-g)) (src/model.c:4451-4452)
         return FAST ? g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.44269504f))
                     : g / (1.0f + expf(-g));

@@ -2,7 +2,11 @@
 //
 // k_moe_route: per token, from the router's 32-bit logits (a matrix product of its own), a softmax over
 // all experts, the `top` experts with the largest score + correction (ties: the lower index), and
-// their weights: the chosen scores (without the correction) over their sum + 1e-20.
+// their weights: the chosen scores (without the correction) over their sum + 1e-20.  Options: the scores are
+// sigmoid(logit), every expert for itself, instead of a softmax; the experts form `groups` equal groups of
+// neighbours, a group's score is the sum of its two largest score + correction, and only experts of the `keep`
+// groups that score highest can be chosen (ties: the lower group); the weights are the chosen scores times a
+// given number instead of their share of their sum.
 // k_moe_up / k_moe_down: the experts' two products token by token, a wave an output column, the
 // weights of the chosen experts streamed: what a few decoded tokens need.  Expert:
 // down(act(up h)), act = relu squared, or gated: down(silu(gate h) * (up h)) with the gate's rows before
@@ -16,20 +20,53 @@
 #define MOE_MAX_TOP 64      // lane j of the routing wave keeps the j-th choice
 
 __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* __restrict__ wts, const float* __restrict__ logits,
-                                                  const float* __restrict__ correction, int ld, int n, int top) {
+                                                  const float* __restrict__ correction, int ld, int n, int top, int sigmoid,
+                                                  int groups, int keep, float weight_scale) {
     __shared__ float z[MOE_MAX_EXPERTS];
+    __shared__ float gsc[MOE_MAX_EXPERTS];          // a group's score; then 1 if its experts can be chosen, else 0
     const int t = blockIdx.x, lane = threadIdx.x;
     for (int e = lane; e < n; e += 64) z[e] = logits[(size_t)t * ld + e];
     __syncthreads();
-    float m = -INFINITY;
-    for (int e = lane; e < n; e += 64) m = fmaxf(m, z[e]);
-    m = wave_max(m);
-    float l = 0.f;
-    for (int e = lane; e < n; e += 64) l += expf(z[e] - m);
-    l = wave_sum(l);
+    if (sigmoid) {
+        for (int e = lane; e < n; e += 64) z[e] = 1.0f / (1.0f + expf(-z[e]));      // the scores
+    } else {
+        float m = -INFINITY;
+        for (int e = lane; e < n; e += 64) m = fmaxf(m, z[e]);
+        m = wave_max(m);
+        float l = 0.f;
+        for (int e = lane; e < n; e += 64) l += expf(z[e] - m);
+        l = wave_sum(l);
+        __syncthreads();
+        for (int e = lane; e < n; e += 64) z[e] = expf(z[e] - m) / l;       // the scores
+    }
     __syncthreads();
-    for (int e = lane; e < n; e += 64) z[e] = expf(z[e] - m) / l;       // the scores
-    __syncthreads();
+    const int per = n / groups;
+    if (groups > 1) {
+        for (int g = lane; g < groups; g += 64) {
+            float a = -INFINITY, b = -INFINITY;         // the group's two largest choice scores
+            for (int e = g * per; e < (g + 1) * per; ++e) {
+                float c = z[e] + correction[e];
+                if (!(c == c)) c = -INFINITY;
+                if (c > a) { b = a; a = c; } else if (c > b) b = c;
+            }
+            gsc[g] = per > 1 ? a + b : a;
+        }
+        __syncthreads();
+        float mine_g[MOE_MAX_EXPERTS / 64];
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i) {
+            const int g = lane + 64 * i;
+            int rank = 0;
+            if (g < groups)
+                for (int o = 0; o < groups; ++o) rank += (gsc[o] > gsc[g] || (gsc[o] == gsc[g] && o < g)) ? 1 : 0;
+            mine_g[i] = rank < keep ? 1.f : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < MOE_MAX_EXPERTS / 64; ++i)
+            if (lane + 64 * i < groups) gsc[lane + 64 * i] = mine_g[i];
+        __syncthreads();
+    }
     // `top` passes of: the largest score + correction not yet taken, the lower index on a tie.  A score
     // that is no number (the row of a request that does not exist, whose state is whatever memory held)
     // counts as the smallest, so that every pass still finds an expert that exists.
@@ -42,6 +79,7 @@ __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* 
         for (int e = lane; e < n; e += 64) {
             const float s = z[e];
             if (s < -0.5f) continue;        // taken: stored as -(s) - 1
+            if (groups > 1 && gsc[e / per] == 0.f) continue;       // its group is out
             float c = s + correction[e];
             if (!(c == c)) c = -INFINITY;
             if (at == n || c > best || (c == best && e < at)) { best = c; at = e; }
@@ -63,17 +101,20 @@ __global__ __launch_bounds__(64) void k_moe_route(int* __restrict__ idx, float* 
     }
     if (lane < top) {
         idx[(size_t)t * top + lane] = mine;
-        wts[(size_t)t * top + lane] = mine_s / (total + 1e-20f);
+        wts[(size_t)t * top + lane] = weight_scale > 0.f ? mine_s * weight_scale : mine_s / (total + 1e-20f);
     }
 }
 
 extern "C" int xr_moe_route(int* idx, float* wts, const float* logits, const float* correction, int T, int ld, int n, int top,
-                            hipStream_t stream) {
+                            int sigmoid, int groups, int keep, float weight_scale, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && ld >= n, "moe_route: bad sizes T=%d ld=%d", T, ld);
     XR_REQUIRE(n >= 1 && n <= MOE_MAX_EXPERTS && top >= 1 && top <= n && top <= MOE_MAX_TOP,
                "moe_route: %d experts (at most %d), %d chosen (at most %d)", n, MOE_MAX_EXPERTS, top, MOE_MAX_TOP);
+    XR_REQUIRE(groups >= 1 && n % groups == 0 && keep >= 1 && keep <= groups && top <= keep * (n / groups),
+               "moe_route: %d experts in %d groups of which %d are kept cannot give %d choices", n, groups, keep, top);
+    XR_REQUIRE(weight_scale >= 0.f, "moe_route: weight scale %g (0: the chosen scores' shares of their sum)", (double)weight_scale);
     if (T == 0) return XR_OK;
-    k_moe_route<<<T, 64, 0, stream>>>(idx, wts, logits, correction, ld, n, top);
+    k_moe_route<<<T, 64, 0, stream>>>(idx, wts, logits, correction, ld, n, top, sigmoid, groups, keep, weight_scale);
     XR_CHECK_LAUNCH("moe_route");
     return XR_OK;
 }

@@ -19,7 +19,7 @@ from . import build as _build
 XR_F32, XR_BF16 = 0, 1
 _CODE = {torch.float32: XR_F32, torch.bfloat16: XR_BF16}
 # activations of a gated feed-forward, by the code the kernels know them under (XR_ACT_* of common.h)
-GATE_ACTIVATIONS = {"silu": 0, "clamped_swish": 1}
+GATE_ACTIVATIONS = {"silu": 0, "clamped_swish": 1, "gelu_tanh": 2}
 # gates that take a number of their own (``param``) and shape both branches (``gate_value`` of common.h)
 SHAPED_GATES = {"clamped_swish"}
 NORM_GATES = {"silu": 0, "sigmoid": 1}                  # XR_GATE_SILU / XR_GATE_SIGMOID of sequence_kernels.hip
@@ -59,7 +59,12 @@ _PROTOS = {
     "xr_gemm_bf16": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p, _sz, _p, _p, _p],
     "xr_pack_weight": [_p, _p, _i, _i, _p],
     "xr_rope_table": [_p, _p, _p, _i, _i, _f, _p],
-    "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _p, _p],
+    "xr_attention_ref": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _i, _p, _p, _p],
+    "xr_attn_extra_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p, _p, _i, _p],
+    "xr_decay_prepare": [_p, _i, _i, _i, _i, _i, _f, _p, _p, _p],
+    "xr_head_gate": [_p, _p, _i, _i, _i, _i, _i, _p],
+    "xr_pair_combine": [_p, _p, _p, _p, _p, _f, _f, _f, _i, _i, _i, _i, _p],
+    "xr_add_rows": [_p, _p, _p, _f, _i, _i, _p],
     "xr_dyt_step": [_p, _p, _p, _p, _f, _f, _p, _p, _p, _f, _p, _i, _i, _i, _i, _i, _p],
     "xr_token_shift": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_head_rmsnorm": [_p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _f, _f, _i, _p],
@@ -77,12 +82,12 @@ _PROTOS = {
     "xr_streams_sum": [_p, _p, _i, _i, _i, _p],
     "xr_streams_step": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _f, _i, _p],
     "xr_latent_prepare": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _f, _i, _p],
-    "xr_moe_route": [_p, _p, _p, _p, _i, _i, _i, _i, _p],
+    "xr_moe_route": [_p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _f, _p],
     "xr_moe_experts_grouped": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p],
     "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
     "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
-    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p],
+    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_attention_pool_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
@@ -90,7 +95,7 @@ _PROTOS = {
 }
 
 CONV_ACTIVATIONS = {None: 0, "none": 0, "silu": 1}      # XR_CONV_* of sequence_kernels.hip
-RECURRENCES = {"retention": 0, "delta": 1, "wkv": 2}    # XR_REC_* of recurrent_kernels.hip
+RECURRENCES = {"retention": 0, "delta": 1, "wkv": 2, "gla": 3, "delta_channel": 4}    # XR_REC_* of recurrent_kernels.hip
 ROW_ACTIVATIONS = {"silu": 1, "tanh": 2}                # what act_rows_ applies in place
 EXPERT_ACTIVATIONS = {"relu2": 0, "swiglu": 1}          # MOE_ACT_* of moe_kernels.hip
 
@@ -594,9 +599,15 @@ class Ops:
         return q
 
     def attention(self, q, k_cache, v_cache, ctx, group: int, H: int, Hk: int, D: int, page_size: int,
-                  scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  scale: float, window: Optional[int] = None, slopes: Optional[torch.Tensor] = None,
+                  chunk: Optional[int] = None, keep_first: int = 0, sinks: Optional[torch.Tensor] = None,
+                  v_head_dim: Optional[int] = None) -> torch.Tensor:
         """Causal attention of every token of the step over its request's cached keys and values.
         ``slopes`` (32-bit ``[H]``): ``slopes[h] * (i - j)`` is taken off the score of query i and key j.
+        ``window``: a position reads the last ``window`` keys; ``chunk``: it reads the keys of its own chunk of
+        ``chunk`` positions, counted from 0; ``keep_first``: the first so many keys are read whatever the window.
+        ``sinks`` (32-bit ``[H]``): the softmax's denominator also holds ``exp(sinks[h])``, an entry without key
+        or value.  ``v_head_dim``: the size of a value where it is not the keys' (``[T, H * v_head_dim]`` comes back).
 
         bfloat16 runs on the matrix cores (head sizes in steps of 16 up to 256, pages of at least
         16 positions); float32, and what the MFMA kernel does not take, runs the 32-bit kernel.
@@ -609,29 +620,97 @@ class Ops:
             raise KernelError("attention: queries and cache differ in dtype")
         if H % Hk:
             raise KernelError(f"attention: {H} query heads are not a multiple of {Hk} key/value heads")
-        out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
-        if slopes is not None:
-            self._dev(slopes)
-            if slopes.dtype != torch.float32 or slopes.numel() != H or not slopes.is_contiguous():
-                raise KernelError(f"attention: the slopes must be float32 [{H}]")
-        if self.use_mfma and q.dtype == torch.bfloat16 and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16:
+        Dv = int(v_head_dim) if v_head_dim is not None else D
+        out = torch.empty((T, H * Dv), dtype=q.dtype, device=q.device)
+        for name, t in (("slopes", slopes), ("sinks", sinks)):
+            if t is not None:
+                self._dev(t)
+                if t.dtype != torch.float32 or t.numel() != H or not t.is_contiguous():
+                    raise KernelError(f"attention: the {name} must be float32 [{H}]")
+        if chunk and window:
+            raise KernelError("attention: a layer reads a window or its chunk, not both")
+        if (self.use_mfma and q.dtype == torch.bfloat16 and D == Dv and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16):
+            # What is no key of the window (or chunk) enters the same softmax as a partial result of its own: the
+            # sink, and the first keys that the window has passed; the kernels' merge adds it to the key ranges'.
+            extra = sinks is not None or keep_first > 0
             lib = self.attention_lib(D)
-            plan = ctx.attention_plan(group, H // Hk, window, Hk, page_size)
+            from ..engine.batch import Chunked
+            plan = ctx.attention_plan(group, H // Hk, Chunked(int(chunk)) if chunk else window, Hk, page_size, extra_slot=extra)
             part_o = part_ml = None
             if plan.n_slots:
                 part_o = torch.empty((plan.n_slots, Hk, 32, D), dtype=torch.float32, device=q.device)
                 part_ml = torch.empty((plan.n_slots, Hk, 32, 2), dtype=torch.float32, device=q.device)
+            if extra:
+                self.lib.check(self.lib.xr_attn_extra_partial(
+                    part_o.data_ptr(), part_ml.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                    plan.extras.data_ptr(), plan.n_extras, block_table.data_ptr(), block_table.stride(0), H, Hk, D, page_size,
+                    float(scale), int(window or 0), int(chunk or 0), int(keep_first), _ptr(sinks), _ptr(slopes),
+                    dtype_code(q.dtype), _stream()))
             lib.check(lib.xr_attention_mfma(
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(window or 0), _ptr(slopes), _stream()))
+                float(scale), int(window or 0), int(chunk or 0), _ptr(slopes), _stream()))
             return out
         self.lib.check(self.lib.xr_attention_ref(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
-            req_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), T, H, Hk, D, page_size,
-            float(scale), int(window or 0), dtype_code(q.dtype), _ptr(slopes), _stream()))
+            req_of_token.data_ptr(), block_table.data_ptr(), block_table.stride(0), T, H, Hk, D, Dv, page_size,
+            float(scale), int(window or 0), int(chunk or 0), int(keep_first), dtype_code(q.dtype), _ptr(slopes),
+            _ptr(sinks), _stream()))
         return out
+
+    def head_gate_(self, o: torch.Tensor, g: torch.Tensor, H: int, Dv: int) -> None:
+        """``o[t, h, :] *= sigmoid(g[t, h])`` in place: ``o [T, H * Dv]`` contiguous, ``g`` a 32-bit view ``[T, H]``."""
+        self._dev(o, g)
+        self._contig(o, "head_gate_ rows")
+        T = o.shape[0]
+        if tuple(o.shape) != (T, H * Dv) or g.dtype != torch.float32 or tuple(g.shape) != (T, H) or g.stride(1) != 1:
+            raise KernelError(f"head_gate_: rows [{T}, {H * Dv}] and a float32 gate view [{T}, {H}] are needed")
+        self.lib.check(self.lib.xr_head_gate(o.data_ptr(), g.data_ptr(), T, H, Dv, g.stride(0), dtype_code(o.dtype), _stream()))
+
+    def decay_prepare_(self, x: torch.Tensor, H: int, D: int, form: str, tau: float = 1.0,
+                       a_log: Optional[torch.Tensor] = None, dt_bias: Optional[torch.Tensor] = None) -> None:
+        """In place on a 32-bit view ``x [T, H * D]``: the decays a token, head and key channel of a recurrence.
+        ``form`` "sigmoid_root": ``sigmoid(x)^(1 / tau)``; "exp_softplus": ``exp(-exp(a_log[h]) * softplus(x + dt_bias[h, c]))``."""
+        self._dev(x, a_log, dt_bias)
+        forms = {"sigmoid_root": 0, "exp_softplus": 1}
+        if form not in forms:
+            raise KernelError(f"decay_prepare_: form {form!r} (known: {sorted(forms)})")
+        if x.dtype != torch.float32 or x.dim() != 2 or x.stride(1) != 1 or x.shape[1] != H * D:
+            raise KernelError(f"decay_prepare_: x must be a float32 view [rows, {H * D}] with unit column stride")
+        if form == "exp_softplus" and (a_log is None or dt_bias is None or a_log.dtype != torch.float32 or dt_bias.dtype != torch.float32
+                                       or a_log.numel() != H or dt_bias.numel() != H * D):
+            raise KernelError(f"decay_prepare_: float32 A_log [{H}] and dt_bias [{H * D}] are needed")
+        self.lib.check(self.lib.xr_decay_prepare(x.data_ptr(), x.shape[0], H, D, x.stride(0), forms[form], float(tau),
+                                                 _ptr(a_log), _ptr(dt_bias), _stream()))
+
+    def pair_combine_(self, x: torch.Tensor, y_left: torch.Tensor, y_right: torch.Tensor, a_left: float, a_right: float,
+                      w_left: Optional[torch.Tensor] = None, w_right: Optional[torch.Tensor] = None, eps: float = 0.0) -> None:
+        """``x += a_left f(y_left) + a_right f(y_right)`` for 32-bit rows ``[T, E]``; with the weights, ``f`` is a row
+        over its root mean square (eps inside the root) times the side's weight ``[E]``, else the identity."""
+        self._dev(x, y_left, y_right, w_left, w_right)
+        T, E = y_left.shape
+        if (x.dtype != torch.float32 or x.stride(1) != 1 or tuple(x.shape) != (T, E)
+                or any(t.dtype != torch.float32 or tuple(t.shape) != (T, E) or not t.is_contiguous() for t in (y_left, y_right))):
+            raise KernelError(f"pair_combine_: x and both results must be float32 [{T}, {E}]")
+        normed = w_left is not None
+        if normed and any(w is None or w.dtype != torch.float32 or w.numel() != E or not w.is_contiguous() for w in (w_left, w_right)):
+            raise KernelError(f"pair_combine_: the sides' norm weights must be float32 [{E}]")
+        self.lib.check(self.lib.xr_pair_combine(x.data_ptr(), y_left.data_ptr(), y_right.data_ptr(), _ptr(w_left), _ptr(w_right),
+                                                float(a_left), float(a_right), float(eps), T, E, x.stride(0), 1 if normed else 0,
+                                                _stream()))
+
+    def add_rows_(self, x: torch.Tensor, v: torch.Tensor, y: Optional[torch.Tensor] = None, scale: float = 1.0) -> None:
+        """``x[t] += scale * y[t] + v`` for 32-bit contiguous rows ``[T, E]`` and a 32-bit vector ``v [E]`` (``y`` absent:
+        the vector alone)."""
+        self._dev(x, v, y)
+        self._contig(x, "add_rows_ x")
+        T, E = x.shape
+        if x.dtype != torch.float32 or v.dtype != torch.float32 or v.numel() != E or not v.is_contiguous():
+            raise KernelError(f"add_rows_: x must be float32 rows and v float32 [{E}]")
+        if y is not None and (y.dtype != torch.float32 or tuple(y.shape) != (T, E) or not y.is_contiguous()):
+            raise KernelError(f"add_rows_: y must be contiguous float32 [{T}, {E}]")
+        self.lib.check(self.lib.xr_add_rows(x.data_ptr(), _ptr(y), v.data_ptr(), float(scale), T, E, _stream()))
 
     def attention_lib(self, D: int) -> "_Lib":
         """The MFMA attention library for head size ``D`` (compiled at first use)."""
@@ -640,7 +719,7 @@ class Ops:
             unit = f"attn_d{D}"
             path = _build.find_built(unit) or _build.build_unit(unit)
             lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _p, _p,
-                                                    _i, _i, _i, _i, _f, _i, _p, _p]})
+                                                    _i, _i, _i, _i, _f, _i, _i, _p, _p]})
             self._attn_libs[D] = lib
         return lib
 
@@ -998,16 +1077,24 @@ class Ops:
             self.linear(a[:, g * a_width:g * a_width + K], w[g], out=out[:, g * out_width:g * out_width + N])
 
     # -- mixture of experts ------------------------------------------------------------
-    def moe_route(self, h: torch.Tensor, router, correction: torch.Tensor, top: int):
+    def moe_route(self, h: torch.Tensor, router, correction: torch.Tensor, top: int, **how):
         """``(experts [T, top] int32, weights [T, top] float32)``: 32-bit logits ``h @ router [n, E]^T`` (a matrix
         product with 32-bit accumulation and a 32-bit result; ``router`` in ``h``'s dtype, a matrix or a
         ``PackedWeight``), a softmax over all experts, the ``top`` largest of score + ``correction`` (the lower
         index on a tie), weights = the chosen scores over their sum + 1e-20."""
         logits = self.linear(h, router, out_dtype=torch.float32)
-        return self.route_logits(logits, correction, top)
+        return self.route_logits(logits, correction, top, **how)
 
-    def route_logits(self, logits: torch.Tensor, correction: torch.Tensor, top: int):
-        """``moe_route`` from the 32-bit logits ``[T, n]``."""
+    def route_logits(self, logits: torch.Tensor, correction: torch.Tensor, top: int, scores: str = "softmax",
+                     groups: int = 1, keep_groups: int = 1, weight_scale: Optional[float] = None):
+        """``moe_route`` from the 32-bit logits ``[T, n]``.  ``scores`` "sigmoid": every expert's score is the sigmoid
+        of its logit.  ``groups`` > 1: the experts form that many equal groups of neighbours, a group scores the
+        sum of its two largest score + correction, and only the ``keep_groups`` best groups' experts can be chosen.
+        ``weight_scale``: the weights are the chosen scores times it instead of their shares of their sum."""
+        if scores not in ("softmax", "sigmoid"):
+            raise KernelError(f"route_logits: scores {scores!r} (softmax or sigmoid)")
+        if weight_scale is not None and not weight_scale > 0:
+            raise KernelError(f"route_logits: weight scale {weight_scale} must be positive")
         self._dev(logits, correction)
         if logits.dtype != torch.float32 or logits.dim() != 2 or logits.stride(1) != 1:
             raise KernelError("route_logits: logits must be float32 [rows, experts] with unit column stride")
@@ -1017,7 +1104,8 @@ class Ops:
         idx = torch.empty((T, top), dtype=torch.int32, device=logits.device)
         wts = torch.empty((T, top), dtype=torch.float32, device=logits.device)
         self.lib.check(self.lib.xr_moe_route(idx.data_ptr(), wts.data_ptr(), logits.data_ptr(), correction.data_ptr(), T,
-                                             logits.stride(0), n, int(top), _stream()))
+                                             logits.stride(0), n, int(top), 1 if scores == "sigmoid" else 0, int(groups),
+                                             int(keep_groups), float(weight_scale or 0.0), _stream()))
         return idx, wts
 
     def table_route(self, table: torch.Tensor, ids: torch.Tensor, n_experts: int):
@@ -1087,18 +1175,19 @@ class Ops:
     def delta_prepare_(self, q, k, b, a, a_log, dt_bias, G: int, H: int, D: int, q_scale: float, unit_eps: float) -> None:
         """In place on 32-bit views (``q`` and ``k`` with one row stride, ``b`` and ``a`` with one):
         query and key heads become unit vectors (queries times ``q_scale``), ``b`` becomes
-        ``sigmoid(b)``, ``a`` becomes ``exp(-exp(a_log) * softplus(a + dt_bias))``."""
+        ``sigmoid(b)``, ``a`` becomes ``exp(-exp(a_log) * softplus(a + dt_bias))`` (``a`` absent: the decays are
+        made elsewhere, by ``decay_prepare_`` for one a key channel)."""
         self._dev(q, k, b, a, a_log, dt_bias)
-        views = (q, k, b, a)
+        views = [t for t in (q, k, b, a) if t is not None]
         if (any(v.dtype != torch.float32 or v.stride(1) != 1 for v in views) or q.stride(0) != k.stride(0)
-                or b.stride(0) != a.stride(0)):
+                or (a is not None and b.stride(0) != a.stride(0))):
             raise KernelError("delta_prepare_: q and k, and b and a, must be float32 views with one row stride each")
-        if tuple(q.shape[1:]) != (G * D,) or tuple(k.shape[1:]) != (G * D,) or b.shape[1] != H or a.shape[1] != H:
+        if tuple(q.shape[1:]) != (G * D,) or tuple(k.shape[1:]) != (G * D,) or b.shape[1] != H or (a is not None and a.shape[1] != H):
             raise KernelError("delta_prepare_: view widths do not fit the heads")
-        if a_log.dtype != torch.float32 or dt_bias.dtype != torch.float32 or a_log.numel() != H or dt_bias.numel() != H:
+        if a is not None and (a_log.dtype != torch.float32 or dt_bias.dtype != torch.float32 or a_log.numel() != H or dt_bias.numel() != H):
             raise KernelError(f"delta_prepare_: A_log and dt_bias must be float32 [{H}]")
-        self.lib.check(self.lib.xr_delta_prepare(q.data_ptr(), k.data_ptr(), b.data_ptr(), a.data_ptr(), a_log.data_ptr(),
-                                                 dt_bias.data_ptr(), q.shape[0], G, H, D, q.stride(0), b.stride(0),
+        self.lib.check(self.lib.xr_delta_prepare(q.data_ptr(), k.data_ptr(), b.data_ptr(), _ptr(a), _ptr(a_log) if a is not None else None,
+                                                 _ptr(dt_bias) if a is not None else None, q.shape[0], G, H, D, q.stride(0), b.stride(0),
                                                  float(q_scale), float(unit_eps), _stream()))
 
     @staticmethod
@@ -1117,6 +1206,8 @@ class Ops:
         S <- S + k u^T`` with ``beta``/``gate [T, H]``; ``o = S^T q`` after the update in both.  "wkv":
         ``o = (S + diag(u) k v^T)^T q`` before the update ``S <- diag(w) S + k v^T``, with ``w = exp(-exp(x))``
         a token, head and key channel from ``gate`` = x ``[T, H * D]`` and the bonus ``decay`` = u ``[H, D]``.
+        "gla": ``S <- diag(w) S + k v^T`` with the decays ``gate`` = w ``[T, H * D]`` as they are, read out after the
+        update; "delta_channel": the delta rule with a decay a key channel, ``gate`` = w ``[T, H * D]``, ``beta [T, H]``.
         ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride.  ``activation`` "silu":
         q, k and v pass SiLU on their way into the kernel (the views themselves stay as they are)."""
         if activation not in (None, "silu"):
@@ -1126,7 +1217,7 @@ class Ops:
         self._dev(q, k, v, state, beta, gate, decay)
         views, gates = (q, k, v), [t for t in (beta, gate) if t is not None]
         if (any(t.dtype != torch.float32 or t.stride(1) != 1 for t in list(views) + gates)
-                or len({t.stride(0) for t in views}) != 1 or len({t.stride(0) for t in gates}) > 1):
+                or len({t.stride(0) for t in views}) != 1 or (kind == "delta" and len({t.stride(0) for t in gates}) > 1)):
             raise KernelError("linear_recurrence: q, k and v, and the gates, must be float32 views with one row stride each")
         T = q.shape[0]
         if tuple(q.shape) != (T, G * D) or tuple(k.shape) != (T, G * D) or tuple(v.shape) != (T, H * Dv):
@@ -1140,6 +1231,12 @@ class Ops:
         if kind == "delta":
             if beta is None or gate is None or tuple(beta.shape) != (T, H) or tuple(gate.shape) != (T, H):
                 raise KernelError("linear_recurrence: the delta rule needs beta and gate [T, H]")
+        elif kind == "delta_channel":
+            if beta is None or gate is None or tuple(beta.shape) != (T, H) or tuple(gate.shape) != (T, H * D) or activation is not None:
+                raise KernelError(f"linear_recurrence: the delta rule with channel decays needs beta [T, {H}] and decays [T, {H * D}]")
+        elif kind == "gla":
+            if G != H or beta is not None or activation is not None or gate is None or tuple(gate.shape) != (T, H * D):
+                raise KernelError(f"linear_recurrence: gla needs a key head a head and decays [T, {H * D}]")
         elif kind == "wkv":
             if (G != H or beta is not None or activation is not None or gate is None or tuple(gate.shape) != (T, H * D)
                     or decay is None or decay.dtype != torch.float32 or decay.numel() != H * D or not decay.is_contiguous()):
@@ -1151,17 +1248,18 @@ class Ops:
         # chunk's last state through the chunk's decays alone: one number a head, or their product channel by
         # channel; a chunk's sum from zero and that add up); the delta rule's chain cannot be cut.
         chunk_len, n_chunks, scratch, prod = 0, 0, None, None
-        if kind in ("retention", "wkv") and ctx.max_q_len >= self.RETENTION_CHUNKED_FROM:
+        if kind in ("retention", "wkv", "gla") and ctx.max_q_len >= self.RETENTION_CHUNKED_FROM:
             n = -(-ctx.max_q_len // self.RETENTION_CHUNK)
             if ctx.B * n <= 4096:
                 chunk_len, n_chunks = self.RETENTION_CHUNK, n
                 scratch = torch.empty((ctx.B * n,) + tuple(state.shape[1:]), dtype=torch.float32, device=q.device)
-                if kind == "wkv":
+                if kind in ("wkv", "gla"):
                     prod = torch.empty((ctx.B * n, H, rows.value * lanes.value), dtype=torch.float32, device=q.device)
         self.lib.check(self.lib.xr_linear_recurrence(out.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), _ptr(beta),
                                                      _ptr(gate), _ptr(decay), state.data_ptr(), ctx.cu_q.data_ptr(),
                                                      ctx.slots.data_ptr(), ctx.B, H, G, D, Dv, q.stride(0),
-                                                     gates[0].stride(0) if gates else 0, RECURRENCES[kind],
+                                                     gate.stride(0) if gate is not None else 0,
+                                                     beta.stride(0) if beta is not None else 0, RECURRENCES[kind],
                                                      chunk_len, n_chunks, _ptr(scratch), _ptr(prod), 1 if activation else 0, _stream()))
         return out
 
@@ -1235,7 +1333,7 @@ class Ops:
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), table.data_ptr(), table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(size), None, _stream()))
+                float(scale), int(size), 0, None, _stream()))
             return out
         self.lib.check(self.lib.xr_attention_pooled(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(pk) if P else None,

@@ -500,6 +500,7 @@ __global__ __launch_bounds__(64) void k_delta_prepare(float* __restrict__ q, flo
     for (int h = threadIdx.x; h < H; h += 64) {
         const size_t i = (size_t)t * ld_g + h;
         b[i] = 1.0f / (1.0f + expf(-b[i]));
+        if (!a) continue;           // (the decays are made elsewhere: one a key channel, say)
         const float z = a[i] + dt_bias[h];
         const float sp = z > 20.0f ? z : log1pf(expf(z));
         a[i] = expf(-expf(a_log[h]) * sp);

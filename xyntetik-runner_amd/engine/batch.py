@@ -43,6 +43,29 @@ class AttentionPlan:
     n_extras: int = 0
 
 
+@dataclass(frozen=True)
+class Chunked:
+    """In place of a window's length: a position reads the keys of its own chunk of ``size`` positions, chunks
+    counted from position 0 of its request."""
+    size: int
+
+
+def first_key(mask, pos: int) -> int:
+    """The first key the query at position ``pos`` reads: ``mask`` None (all), a window's length or a ``Chunked``."""
+    if not mask:
+        return 0
+    if isinstance(mask, Chunked):
+        return pos - pos % mask.size
+    return max(0, pos - mask + 1)
+
+
+def mask_reach(mask) -> Optional[int]:
+    """The most keys a query reads under ``mask`` (None: all)."""
+    if not mask:
+        return None
+    return mask.size if isinstance(mask, Chunked) else int(mask)
+
+
 # The first four are the attention kernels' shapes.  The last three are tuning, not limits: they
 # say how much work gives every one of an MI355X's 256 compute units a workgroup, measured on the
 # 8B shape's attention; on another chip or shape they cost speed, never correctness.
@@ -66,9 +89,11 @@ def key_ranges(tiles: int, share: float) -> int:
     return max(1, min(int(share), tiles // ATTN_MIN_RANGE))
 
 
-def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_heads: int,
+def plan_attention(starts, q_lens, group_size: int, window, n_kv_heads: int,
                    page_size: int = 64, cta_tiles: Optional[int] = None, extra_slot: bool = False):
     """Host side of ``AttentionPlan``: ``(cta_items, items, jobs, n_slots)`` as plain Python ints.
+
+    ``window``: None, a window's length, or a ``Chunked``.
 
     ``cta_tiles`` fixes the most tiles a 128-row item may cover (for measurements); by
     default it follows from how many such items the step has.
@@ -89,7 +114,7 @@ def plan_attention(starts, q_lens, group_size: int, window: Optional[int], n_kv_
     def key_range(s, n, row0, rows):
         tok_lo = row0 // group_size
         tok_hi = min(n - 1, (row0 + rows - 1) // group_size)
-        lo = 0 if not window else max(0, s + tok_lo - window + 1)
+        lo = first_key(window, s + tok_lo)
         lo = (lo // ATTN_TILE) * ATTN_TILE
         hi = s + tok_hi + 1
         return lo, hi, -(-(hi - lo) // ATTN_TILE)
@@ -255,7 +280,7 @@ class StepContext:
         self._plans = {}
         self.shared = {}        # what parts make once a step and share between layers (a rotation's table)
 
-    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
+    def attention_plan(self, group: int, group_size: int, window, n_kv_heads: int,
                        page_size: int = 64, extra_slot: bool = False) -> AttentionPlan:
         """The MFMA attention work list, made once per step and shared by all layers that can."""
         key = (group_size, window, n_kv_heads, page_size, extra_slot)

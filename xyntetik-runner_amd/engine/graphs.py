@@ -22,7 +22,7 @@ import numpy as np
 import torch
 
 from ..cache import NULL_PAGE
-from .batch import ATTN_MIN_RANGE, ATTN_STREAM_SLOTS, ATTN_TILE, AttentionPlan, StepEntry
+from .batch import ATTN_MIN_RANGE, ATTN_STREAM_SLOTS, ATTN_TILE, AttentionPlan, Chunked, StepEntry, mask_reach
 
 BUCKETS = (1, 2, 4, 8, 16, 32, 64, 128, 256, 512)
 SPLITS = (1, 2, 4, 8, 16, 32)
@@ -121,7 +121,7 @@ class StaticDecodeContext:
         raise RuntimeError("this step is recorded as a graph: a part with state reads its rows' slots from "
                            "ctx.slots (on the device), or sets capturable = False to be run eagerly")
 
-    def attention_plan(self, group: int, group_size: int, window: Optional[int], n_kv_heads: int,
+    def attention_plan(self, group: int, group_size: int, window, n_kv_heads: int,
                        page_size: int = 64, extra_slot: bool = False) -> AttentionPlan:
         key = (group_size, window, n_kv_heads, bool(extra_slot))
         if key not in self._plans:
@@ -129,7 +129,7 @@ class StaticDecodeContext:
                 raise RuntimeError("an attention plan was first asked for during graph capture")
             tiles = self.max_tiles
             if tiles is not None and window:
-                tiles = min(tiles, -(-window // ATTN_TILE) + 1)
+                tiles = min(tiles, -(-mask_reach(window) // ATTN_TILE) + 1)
             self._plan_splits[key] = self.S if tiles is None else min(self.S, splits_for(self.B, tiles, n_kv_heads))
             self._plan_keys.append(key)
             self._alloc()
@@ -205,7 +205,9 @@ class StaticDecodeContext:
         jobs = h[base + B * S * 8:base + B * S * 8 + B * 7].reshape(B, 7)
         hi = starts.astype(np.int64) + 1                          # keys [lo, hi)
         lo = np.zeros(B, dtype=np.int64)
-        if window:
+        if isinstance(window, Chunked):
+            lo = starts.astype(np.int64) - starts.astype(np.int64) % window.size
+        elif window:
             lo = np.maximum(0, starts.astype(np.int64) - window + 1)
         lo = (lo // ATTN_TILE) * ATTN_TILE
         tiles = -(-(hi - lo) // ATTN_TILE)

@@ -129,7 +129,7 @@ class Model:
         for i, step in enumerate(order):
             block = self.blocks[step.layer]
             if step.enters:         # (the block before made no input for this one: the stream it would have read is remade here)
-                x = self.injection.forward(ctx, x, x0)
+                x = self.injection.forward(ctx, x, x0, step.pass_index)
             if block.chained:
                 chain = i + 1 < len(order) and not order[i + 1].enters
                 after = self.blocks[order[i + 1].layer].entry_norm() if chain else None

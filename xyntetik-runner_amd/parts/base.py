@@ -85,6 +85,8 @@ class KVSpec:
     layer keeps one mean key and one mean value for every block of P positions, in a
     cache of their own whose group has ``stride`` P (one entry for every ``stride``
     positions a request has filled, never given back while the request lives).
+    ``keep_first``: with a window, the pages of the first so many positions are kept as well for as
+    long as the request lives.
     """
     num_kv_heads: int
     head_dim: int
@@ -92,6 +94,7 @@ class KVSpec:
     v_head_dim: Optional[int] = None
     pooled: Optional[int] = None
     stride: int = 1
+    keep_first: int = 0
 
     @property
     def value_dim(self) -> int:
@@ -225,13 +228,14 @@ class Connection(Part):
 
 class Injection(Part):
     """What remakes the residual stream from itself and the embedding's rows at the start of a pass over a
-    span of layers: ``forward(ctx, x, x0) -> x'`` with ``x`` and the result 32-bit ``[T, E]``; ``x0`` is what
-    ``prepare(ctx, embedded)`` made of the embedding's rows when the step began."""
+    span of layers: ``forward(ctx, x, x0, pass_index) -> x'`` with ``x`` and the result 32-bit ``[T, E]``; ``x0`` is
+    what ``prepare(ctx, embedded)`` made of the embedding's rows when the step began; ``pass_index`` counts the
+    passes from 0."""
 
     def prepare(self, ctx, embedded: torch.Tensor):
         return embedded
 
-    def forward(self, ctx, x: torch.Tensor, x0) -> torch.Tensor:
+    def forward(self, ctx, x: torch.Tensor, x0, pass_index: int = 0) -> torch.Tensor:
         raise NotImplementedError
 
 

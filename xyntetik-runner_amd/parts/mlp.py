@@ -13,7 +13,11 @@ the weights are the chosen scores over their sum) and added up with those weight
 are gated feed-forwards themselves, ``down_e(silu(gate_e(h)) * up_e(h))`` (``activation="swiglu"``); a choice
 without a router, by a table ``[vocab, top]`` of expert numbers that the token's id indexes, every chosen
 expert with the weight ``1 / top`` (``routing="table"``); a shared expert that runs for every token and is
-added to the sum (``shared_size``: its inner width; a gated feed-forward with the SiLU gate).
+added to the sum (``shared_size``: its inner width; a gated feed-forward with the SiLU gate); scores that are
+the sigmoid of each expert's logit instead of a softmax over all (``scores="sigmoid"``); a choice limited to the best
+groups (``groups`` equal groups of neighbouring experts, a group's score the sum of its two largest score +
+correction, ``keep_groups`` groups whose experts can be chosen; the others count as minus infinity); weights that are
+the chosen scores times a number (``weight_scale``) instead of their shares of their sum.
 
 Dense feed-forward: ``down(act(up(h)))`` with an activation over the whole row.  "polynorm":
 ``a N(z) + b N(z^2) + c N(z^3) + e`` with four learned numbers, powers element by element and
@@ -140,7 +144,8 @@ class RoutedExperts(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, num_experts: int, top: int, activation: str = "relu2",
                  router_name: str = "router", correction_name: str = "correction", expert_prefix: str = "e",
                  up_name: str = "up", down_name: str = "down", gate_name: str = "gate", routing: str = "router",
-                 vocab_size: int = 0, table_name: str = "table", shared_size: int = 0, shared_prefix: str = "shared."):
+                 vocab_size: int = 0, table_name: str = "table", shared_size: int = 0, shared_prefix: str = "shared.",
+                 scores: str = "softmax", groups: int = 1, keep_groups: int = 1, weight_scale=None):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"routed experts: activation {activation!r} is not built (known: {list(self.ACTIVATIONS)})")
         if routing not in self.ROUTINGS:
@@ -159,6 +164,17 @@ class RoutedExperts(FeedForward):
                              f"not {num_experts} and {top}")
         self.hidden_size, self.intermediate_size = int(hidden_size), int(intermediate_size)
         self.num_experts, self.top = int(num_experts), int(top)
+        groups, keep_groups = int(groups), int(keep_groups)
+        if scores not in ("softmax", "sigmoid"):
+            raise ValueError(f"routed experts: scores {scores!r} (softmax or sigmoid)")
+        if (groups < 1 or self.num_experts % groups or not (1 <= keep_groups <= groups)
+                or self.top > keep_groups * (self.num_experts // groups)):
+            raise ValueError(f"routed experts: {num_experts} experts in {groups} groups of which {keep_groups} are kept "
+                             f"cannot give {top} choices a token")
+        if weight_scale is not None and not float(weight_scale) > 0.0:
+            raise ValueError(f"routed experts: weight scale {weight_scale} must be positive")
+        self.how = dict(scores=scores, groups=groups, keep_groups=keep_groups,
+                        weight_scale=float(weight_scale) if weight_scale is not None else None)
         self.names = (router_name, correction_name, expert_prefix, up_name, down_name)
 
     def param_specs(self) -> Dict[str, ParamSpec]:
@@ -201,7 +217,7 @@ class RoutedExperts(FeedForward):
         if self.routing == "table":
             idx, wts = ops.table_route(self.table, ctx.token_ids, self.num_experts)
         else:
-            idx, wts = ops.moe_route(h, self.router, self.correction, self.top)
+            idx, wts = ops.moe_route(h, self.router, self.correction, self.top, **self.how)
         out = ops.moe_experts(h, self.w_up, self.w_down, idx, wts, out=out, accumulate=accumulate, activation=self.activation)
         if self.shared is not None:
             self.shared.forward_add(ctx, h, out)

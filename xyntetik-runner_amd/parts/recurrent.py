@@ -16,7 +16,16 @@ and ``v`` (H heads of Dv) each pass a short causal convolution over time and SiL
 unit vectors ``x / sqrt(sum(x^2) + 1e-6)``, q also times ``D^-1/2``; ``beta = sigmoid(Wb h)`` and
 ``g = exp(-exp(A_log_h) * softplus(Wa h + dt_bias_h))`` a head; ``S <- g S; u = beta (v - S^T k);
 S <- S + k u^T``.  The read-out is divided by its root mean square, times a weight over Dv that
-the heads share, times ``silu(Wg h)``, then ``Wo``.
+the heads share, times ``silu(Wg h)``, then ``Wo``.  Options: a decay a head *and key channel*
+(``decay="channel"``: ``g = exp(-exp(A_log_h) * softplus(Wa2 (Wa1 h) + dt_bias))`` laid out heads x D, the decay's
+projection in two thin factors whose inner width the stored tensors decide, ``dt_bias`` a number a channel); a gate
+through two thin factors (``gate="low_rank"``: ``Wg2 (Wg1 h)``); the sigmoid instead of SiLU on the gate
+(``gate_activation``).
+
+``GatedLinearAttention``: linear attention with a decay a token, head and key channel.  ``q = Wq h * D^-1/2``,
+``k = Wk h`` (H heads of D), ``v = Wv h`` (H heads of Dv); ``w = sigmoid(Wa2 (Wa1 h) + b)^(1/tau)`` laid out heads x D;
+``S <- diag(w) S + k v^T``, read out after the update.  Every head's read-out is divided by its root mean square,
+times a weight over Dv that the heads share, times ``silu(Wg h)``, then ``Wo``.
 
 ``TimeMixWKV``: time mixing with a decay a token, head and key channel.  Each of r, k, v, g and the
 decay reads a mix of its own of the token's row and the row before, ``h + (h_before - h) mu_s`` (the row
@@ -137,14 +146,98 @@ class Retention(Mixer):
         self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
 
 
+def pad_inner(w1: torch.Tensor, w2: torch.Tensor):
+    """Two thin factors ``w1 [r, E]`` and ``w2 [N, r]`` with the inner side in whole groups of 8 (what the matrix
+    cores take): rows and columns of zeros, which add nothing."""
+    r = int(w1.shape[0])
+    if w2.shape[1] != r:
+        raise ValueError(f"thin factors {tuple(w1.shape)} and {tuple(w2.shape)} do not meet")
+    if r % 8:
+        pad = 8 - r % 8
+        w1 = torch.cat([w1, w1.new_zeros((pad, w1.shape[1]))], dim=0)
+        w2 = torch.cat([w2, w2.new_zeros((w2.shape[0], pad))], dim=1)
+    return w1.contiguous(), w2.contiguous()
+
+
+def _random_rank(E: int) -> int:
+    """The inner width the random-weights mode gives a pair of thin factors; a file may bring any."""
+    return max(4, E // 16)
+
+
+class GatedLinearAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, head_dim: int, v_head_dim: int, tau: float, eps: float,
+                 q_name: str = "q", k_name: str = "k", v_name: str = "v", g_name: str = "g", o_name: str = "o",
+                 a1_name: str = "a1", a2_name: str = "a2", a_bias_name: str = "a2.b", norm_name: str = "norm"):
+        _check_sizes("gated linear attention", num_heads, num_heads, head_dim, v_head_dim)
+        if not float(tau) > 0.0:
+            raise ValueError(f"gated linear attention: tau {tau} must be positive")
+        self.hidden_size, self.num_heads = int(hidden_size), int(num_heads)
+        self.head_dim, self.v_head_dim, self.tau, self.eps = int(head_dim), int(v_head_dim), float(tau), float(eps)
+        self.names = dict(q=q_name, k=k_name, v=v_name, g=g_name, o=o_name, a1=a1_name, a2=a2_name, ab=a_bias_name, norm=norm_name)
+        self.qk_size, self.v_size = self.num_heads * self.head_dim, self.num_heads * self.v_head_dim
+
+    def state_spec(self):
+        from ..csrc.ops import Ops
+        return StateSpec(Ops.recurrence_state_shape(self.num_heads, self.head_dim, self.v_head_dim), torch.float32)
+
+    def param_specs(self) -> Dict[str, ParamSpec]:
+        E, QK, V, n = self.hidden_size, self.qk_size, self.v_size, self.names
+        rank = _random_rank(E)
+        return {n["q"]: ParamSpec((QK, E)), n["k"]: ParamSpec((QK, E)), n["v"]: ParamSpec((V, E)), n["g"]: ParamSpec((V, E)),
+                n["o"]: ParamSpec((E, V)),
+                n["a1"]: ParamSpec((-1, E), random_shape=(rank, E)),
+                n["a2"]: ParamSpec((QK, -1), init="normal:0.5", random_shape=(QK, rank)),
+                # decays between a half and nearly one: a state that lasts tens of tokens, neither one nor all
+                n["ab"]: ParamSpec((QK,), role="vector", init="around:2.0:1.5"),
+                n["norm"]: ParamSpec((self.v_head_dim,), role="vector", init="ones_jitter")}
+
+    def bind(self, tensors, rt) -> None:
+        self.rt = rt
+        n = self.names
+        self.w_in = rt.ops.pack_weight(torch.cat([tensors[n[key]] for key in ("q", "k", "v", "g")], dim=0).contiguous())
+        w1, w2 = pad_inner(tensors[n["a1"]], tensors[n["a2"]])
+        self.w_a1, self.w_a2 = rt.ops.pack_weight(w1), rt.ops.pack_weight(w2)
+        self.b_a = tensors[n["ab"]].float().contiguous()
+        self.w_norm = tensors[n["norm"]].float().contiguous()
+        self.w_out = rt.ops.pack_weight(tensors[n["o"]])
+
+    def _read_out(self, ctx, cache, h):
+        ops = self.rt.ops
+        H, D, Dv, QK, V = self.num_heads, self.head_dim, self.v_head_dim, self.qk_size, self.v_size
+        proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
+        q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
+        ops.rotate_rows_(q, ctx.positions, None, H, D, 0, D ** -0.5)          # (no rotation: the scale alone)
+        w = ops.linear(ops.linear(h, self.w_a1), self.w_a2, bias=self.b_a, out_dtype=torch.float32)
+        ops.decay_prepare_(w, H, D, "sigmoid_root", tau=self.tau)
+        state = cache.state if cache.state is not None else cache.states["mixer"]
+        o = ops.linear_recurrence("gla", q, k, v, state, ctx, H, H, D, Dv, gate=w)
+        return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype)
+
+    def forward(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_f32(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out_dtype=torch.float32)
+
+    def forward_add(self, ctx, cache, h, residual) -> None:
+        self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
+
+
 class GatedDelta(Mixer):
     UNIT_EPS = 1e-6
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int,
                  conv_taps: int, eps: float, q_name: str = "q", k_name: str = "k", v_name: str = "v", b_name: str = "b",
                  a_name: str = "a", a_log_name: str = "A_log", dt_bias_name: str = "dt_bias", norm_name: str = "norm",
-                 g_name: str = "g", o_name: str = "o", conv_suffix: str = ".conv"):
+                 g_name: str = "g", o_name: str = "o", conv_suffix: str = ".conv", decay: str = "head",
+                 gate: str = "full", gate_activation: str = "silu", a1_name: str = "a1", a2_name: str = "a2",
+                 g1_name: str = "g1", g2_name: str = "g2"):
         _check_sizes("gated delta rule", num_heads, num_kv_heads, head_dim, v_head_dim)
+        if decay not in ("head", "channel") or gate not in ("full", "low_rank") or gate_activation not in ("silu", "sigmoid"):
+            raise ValueError(f"gated delta rule: decay {decay!r} (head, channel), gate {gate!r} (full, low_rank), "
+                             f"gate activation {gate_activation!r} (silu, sigmoid)")
+        self.decay_kind, self.gate_kind, self.gate_activation = decay, gate, gate_activation
+        self.thin = dict(a1=a1_name, a2=a2_name, g1=g1_name, g2=g2_name)
         if not (0 <= int(conv_taps) <= 16):          # 0: no convolution (SiLU alone), and no tensors of one
             raise ValueError(f"gated delta rule: {conv_taps} convolution taps (0 to 16)")
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
@@ -171,18 +264,38 @@ class GatedDelta(Mixer):
             if self.conv_taps:
                 specs[n[key] + self.conv_suffix] = ParamSpec((rows, self.conv_taps), role="vector", init="normal:0.6")
         specs[n["b"]] = ParamSpec((H, E))
-        specs[n["a"]] = ParamSpec((H, E))
+        rank, t = _random_rank(E), self.thin
+        if self.decay_kind == "channel":
+            specs[t["a1"]] = ParamSpec((-1, E), random_shape=(rank, E))
+            specs[t["a2"]] = ParamSpec((H * self.head_dim, -1), init="normal:0.5", random_shape=(H * self.head_dim, rank))
+            specs[n["dt_bias"]] = ParamSpec((H * self.head_dim,), role="vector", init="normal:0.5")
+        else:
+            specs[n["a"]] = ParamSpec((H, E))
+            specs[n["dt_bias"]] = ParamSpec((H,), role="vector", init="normal:0.5")
         specs[n["a_log"]] = ParamSpec((H,), role="vector", init="normal:0.5")
-        specs[n["dt_bias"]] = ParamSpec((H,), role="vector", init="normal:0.5")
         specs[n["norm"]] = ParamSpec((self.v_head_dim,), role="vector", init="ones_jitter")
-        specs[n["g"]] = ParamSpec((self.v_size, E))
+        if self.gate_kind == "low_rank":
+            specs[t["g1"]] = ParamSpec((-1, E), random_shape=(rank, E))
+            specs[t["g2"]] = ParamSpec((self.v_size, -1), init="normal:0.5", random_shape=(self.v_size, rank))
+        else:
+            specs[n["g"]] = ParamSpec((self.v_size, E))
         specs[n["o"]] = ParamSpec((E, self.v_size))
         return specs
 
     def bind(self, tensors, rt) -> None:
         self.rt = rt
         n = self.names
-        self.w_in = rt.ops.pack_weight(torch.cat([tensors[n[key]] for key in ("q", "k", "v", "g", "b", "a")], dim=0).contiguous())
+        # one product for everything of the full width: q, k, v first (the convolution's columns), then the
+        # gate (if it is no pair of thin factors), the write strengths, the decays a head (if they are)
+        fused = ["q", "k", "v"] + (["g"] if self.gate_kind == "full" else []) + ["b"] + (["a"] if self.decay_kind == "head" else [])
+        self.w_in = rt.ops.pack_weight(torch.cat([tensors[n[key]] for key in fused], dim=0).contiguous())
+        t = self.thin
+        if self.decay_kind == "channel":
+            w1, w2 = pad_inner(tensors[t["a1"]], tensors[t["a2"]])
+            self.w_a1, self.w_a2 = rt.ops.pack_weight(w1), rt.ops.pack_weight(w2)
+        if self.gate_kind == "low_rank":
+            w1, w2 = pad_inner(tensors[t["g1"]], tensors[t["g2"]])
+            self.w_g1, self.w_g2 = rt.ops.pack_weight(w1), rt.ops.pack_weight(w2)
         if self.conv_taps:
             self.w_conv = torch.cat([tensors[n[key] + self.conv_suffix].float() for key in ("q", "k", "v")], dim=0).contiguous()
         else:       # one tap of weight 1: the kernel's SiLU alone
@@ -199,13 +312,29 @@ class GatedDelta(Mixer):
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         y = ops.causal_conv(proj[:, :C], self.w_conv, cache.states.get("mixer.conv"), ctx, torch.float32, activation="silu")
         q, k, v = y[:, :QK], y[:, QK:2 * QK], y[:, 2 * QK:]
-        gate, b, a = proj[:, C:C + V], proj[:, C + V:C + V + H], proj[:, C + V + H:]
-        ops.delta_prepare_(q, k, b, a, self.a_log, self.dt_bias, G, H, D, D ** -0.5, self.UNIT_EPS)
-        o = ops.linear_recurrence("delta", q, k, v, cache.states["mixer.S"], ctx, H, G, D, Dv, beta=b, gate=a)
-        return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype)
+        at = C
+        if self.gate_kind == "full":
+            gate = proj[:, at:at + V]
+            at += V
+        else:
+            gate = ops.linear(ops.linear(h, self.w_g1), self.w_g2, out_dtype=torch.float32)
+        b = proj[:, at:at + H]
+        if self.decay_kind == "channel":
+            w = ops.linear(ops.linear(h, self.w_a1), self.w_a2, out_dtype=torch.float32)
+            ops.decay_prepare_(w, H, D, "exp_softplus", a_log=self.a_log, dt_bias=self.dt_bias)
+            ops.delta_prepare_(q, k, b, None, None, None, G, H, D, D ** -0.5, self.UNIT_EPS)
+            o = ops.linear_recurrence("delta_channel", q, k, v, cache.states["mixer.S"], ctx, H, G, D, Dv, beta=b, gate=w)
+        else:
+            a = proj[:, at + H:]
+            ops.delta_prepare_(q, k, b, a, self.a_log, self.dt_bias, G, H, D, D ** -0.5, self.UNIT_EPS)
+            o = ops.linear_recurrence("delta", q, k, v, cache.states["mixer.S"], ctx, H, G, D, Dv, beta=b, gate=a)
+        return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
 
     def forward(self, ctx, cache, h):
         return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out)
+
+    def forward_f32(self, ctx, cache, h):
+        return self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out_dtype=torch.float32)
 
     def forward_add(self, ctx, cache, h, residual) -> None:
         self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
@@ -296,3 +425,4 @@ class TimeMixWKV(Mixer):
 register_mixer("retention", Retention)
 register_mixer("wkv_time_mix", TimeMixWKV)
 register_mixer("gated_delta", GatedDelta)
+register_mixer("gated_linear_attention", GatedLinearAttention)
