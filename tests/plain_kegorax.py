@@ -247,6 +247,23 @@ def route(z, correction, top, groups, keep, scale):
     return chosen, s[chosen] * scale
 
 
+def route_margin(z, correction, top, groups, keep):
+    """By how much the choice of ``route`` is decided: the smaller of the gap between the last kept group's score
+    and the next group's, and the gap between the last chosen expert's choice score and the next one's among the
+    kept groups' experts (infinite where there is no next).  A computation in fewer bits may choose otherwise
+    where this is within its rounding."""
+    c = sigmoid(z) + correction
+    n = len(z)
+    per = n // groups
+    gs = np.array([np.sort(c[g * per:(g + 1) * per])[::-1][:2].sum() for g in range(groups)])
+    order = np.argsort(-gs, kind="stable")
+    gap = gs[order[keep - 1]] - gs[order[keep]] if keep < groups else np.inf
+    allowed = np.sort(np.concatenate([c[g * per:(g + 1) * per] for g in order[:keep]]))[::-1]
+    if top < len(allowed):
+        gap = min(gap, allowed[top - 1] - allowed[top])
+    return gap
+
+
 def moe_ff(h, w, p, mlp, choices=None):
     r = mlp["router"]
     groups = r.get("groups") or {"count": 1, "keep": 1}
@@ -255,7 +272,7 @@ def moe_ff(h, w, p, mlp, choices=None):
     for t in range(h.shape[0]):
         chosen, wts = route(logits[t], w[p + "correction"], r["top"], groups["count"], groups["keep"], r["scale"])
         if choices is not None:
-            choices.append((logits[t], chosen))
+            choices.append((logits[t], chosen, route_margin(logits[t], w[p + "correction"], r["top"], groups["count"], groups["keep"])))
         for e, a in zip(chosen, wts):
             q = f"{p}e{e}."
             out[t] += a * ((silu(h[t] @ w[q + "gate"].T) * (h[t] @ w[q + "up"].T)) @ w[q + "down"].T)
@@ -278,7 +295,7 @@ def run_order(cfg):
 
 def forward(cfg, w, tokens, taps=None, choices=None):
     """Logits ``[T, vocab]`` of the whole sequence.  ``taps``: a list that receives the residual stream after
-    every layer run; ``choices``: one that receives (router logits, chosen experts) of every routed token."""
+    every layer run; ``choices``: one that receives (router logits, chosen experts, ``route_margin``) of every routed token."""
     eps = cfg["norm"]["eps"]
     scale = (cfg.get("embedding") or {}).get("scale", 1.0)
     x0 = w["embed"][np.asarray(tokens)] * scale
