@@ -348,7 +348,37 @@ def dinasun_config(width, layers, vocab=32000):
     return cfg
 
 
-DESIGNS = {"suripel": ("Suripel", suripel_config), "sugosun": ("Sugosun", sugosun_config), "dinasun": ("Dinasun", dinasun_config)}
+def kegorax_config(width, layers, vocab=32000):
+    """A Kegorax model of real layer sizes whose layer runs are ``layers``: of every three layers the gated delta rule
+    with a decay a key channel (heads of 128, two heads a key head, four taps), chunked attention with a sink and a gate a
+    head (heads of 128, four query heads a key/value head, chunks of 1,024, half the head rotated) beside gated linear
+    attention (half as many heads of 128), and windowed attention that keeps four tokens (a window of 1,024) beside
+    retention; a gated dense feed-forward of 3.5 x width, but 16 experts of width / 2 (2 a token, from 2 of 4 groups) in
+    the chunked layers; a third of the runs are the second pass over a span in the middle."""
+    again = layers // 3
+    distinct = layers - again
+    H = width // 128
+    dense = {"kind": "dense", "ff": int(width * 3.5)}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 16, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+    att = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
+    half = max(1, H // 2)
+    delta = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": half, "dim": 128, "vdim": 128, "conv": 4}, "mlp": dense}
+    par = {"type": "parallel", "mixer": {"left": dict(att, mask={"size": 1024}, rot={"base": 1e6, "dims": 64}),
+                                         "right": {"heads": half, "dim": 128, "vdim": 128, "tau": 16.0}}, "mlp": moe}
+    par2 = {"type": "parallel_2", "mixer": {"left": dict(att, mask={"size": 1024, "keep_first": 4}),
+                                            "right": {"heads": half, "dim": 128, "vdim": 128,
+                                                      "decay": [1 - 0.06 * 0.75 ** (8 * i / half) for i in range(half)]},
+                                            "left_scale": 0.6, "right_scale": 0.9}, "mlp": dense}
+    cfg = {"architecture": "Kegorax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
+           "layers": [(delta, par, par2)[i % 3] for i in range(distinct)]}
+    if again:
+        start = (distinct - again) // 2
+        cfg["loop"] = {"start": start, "stop": start + again, "times": 2}
+    return cfg
+
+
+DESIGNS = {"suripel": ("Suripel", suripel_config), "sugosun": ("Sugosun", sugosun_config), "dinasun": ("Dinasun", dinasun_config),
+           "kegorax": ("Kegorax", kegorax_config)}
 
 
 def llama_like(width, layers, vocab=32000):
@@ -451,7 +481,7 @@ def main():
                     help="also write the command and the JSON line into FILE (markdown)")
     ap.add_argument("--mixed", type=int, default=0, metavar="N",
                     help="also run N requests with prompts of 128..2048 tokens and 128 decoded tokens each through the scheduler")
-    ap.add_argument("--design", default="", choices=["", "suripel", "sugosun", "dinasun"],
+    ap.add_argument("--design", default="", choices=["", "suripel", "sugosun", "dinasun", "kegorax"],
                     help="instead of the serving benchmark: this design at real layer sizes beside the Llama decoder of equal size")
     ap.add_argument("--design-sizes", default="2048,4096", metavar="LIST", help="widths of the --design models")
     ap.add_argument("--design-layers", type=int, default=12, help="layers of the --design models")

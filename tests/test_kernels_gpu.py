@@ -527,12 +527,14 @@ class FakeCtx:
     def block_table(self, group):
         return self._table
 
-    def attention_plan(self, group, G, window, Hk, page_size=64):
-        cta, items, jobs, n_slots = self._plan_fn(self.starts, self.q_lens, G, window, Hk, page_size,
-                                                  cta_tiles=self.cta_tiles)
+    def attention_plan(self, group, G, window, Hk, page_size=64, extra_slot=False):
+        planned = self._plan_fn(self.starts, self.q_lens, G, window, Hk, page_size, cta_tiles=self.cta_tiles,
+                                extra_slot=extra_slot)
+        cta, items, jobs, n_slots = planned[:4]
         it = torch.tensor([v for i in cta + items for v in i], dtype=torch.int32, device=DEV)
         jb = torch.tensor([v for j in jobs for v in j], dtype=torch.int32, device=DEV) if jobs else None
-        return self._Plan(it, len(items), jb, len(jobs), n_slots, len(cta))
+        ex = torch.tensor([v for x in planned[4] for v in x], dtype=torch.int32, device=DEV) if extra_slot else None
+        return self._Plan(it, len(items), jb, len(jobs), n_slots, len(cta), ex, len(planned[4]) if extra_slot else 0)
 
 
 def scatter_pages(n_req_lens, page_size, seed):

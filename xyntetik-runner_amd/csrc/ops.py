@@ -635,7 +635,9 @@ class Ops:
             extra = sinks is not None or keep_first > 0
             lib = self.attention_lib(D)
             from ..engine.batch import Chunked
-            plan = ctx.attention_plan(group, H // Hk, Chunked(int(chunk)) if chunk else window, Hk, page_size, extra_slot=extra)
+            mask = Chunked(int(chunk)) if chunk else window
+            plan = (ctx.attention_plan(group, H // Hk, mask, Hk, page_size, extra_slot=True) if extra
+                    else ctx.attention_plan(group, H // Hk, mask, Hk, page_size))
             part_o = part_ml = None
             if plan.n_slots:
                 part_o = torch.empty((plan.n_slots, Hk, 32, D), dtype=torch.float32, device=q.device)
