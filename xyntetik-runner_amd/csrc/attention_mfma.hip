@@ -66,7 +66,14 @@ struct AttnArgs {
     int window;             // > 0: a row at position p reads the keys from p - window + 1 on
     int chunk;              // > 0: it reads from p - p mod chunk on (its own chunk of positions, counted from 0)
     const float* slopes;    // [H], or null: slopes[h] * (i - j) is taken off the score of query i and key j
+    const float* sinks;     // [H], or null: the softmax's denominator also holds exp(sinks[h]), an entry without key or value;
+                            // it is added where a row's result is finished: by the item that writes the output, or by the merge
 };
+
+// a finished row's sum with the sink's share: the sums are in units of 2^m (m the row's reference in units of log2)
+__device__ inline float with_sink(const float* sinks, int h, float m, float l) {
+    return sinks ? l + __builtin_amdgcn_exp2f(sinks[h] * 1.44269504f - m) : l;
+}
 
 __device__ inline uint4 ldg16(const bf16_t* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ inline bf16x8 as_bf16x8(uint4 v) {
@@ -226,8 +233,9 @@ struct CtaShape {
 // a row block's result: the final output, or the partial result of a key range
 __device__ inline void cta_write_out(const AttnArgs& a, const f32x16 (&o)[DB], float m, float l, bool row_ok, int t, int h,
                                      int kvh, int lr, int lg, int slot) {
-    const float inv = l > 0.f ? 1.0f / l : 0.f;
     if (!row_ok) return;
+    if (slot < 0) l = with_sink(a.sinks, h, m, l);
+    const float inv = l > 0.f ? 1.0f / l : 0.f;
     if (slot < 0) {
         bf16_t* op = a.out + ((size_t)t * a.H + h) * HD;
 #pragma unroll
@@ -981,8 +989,9 @@ __global__ __launch_bounds__(64 * STREAM_WAVES) void k_attn_stream(AttnArgs a) {
             acc.x += f * v.x; acc.y += f * v.y; acc.z += f * v.z; acc.w += f * v.w;
             lsum += f * lw;
         }
-        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
         const int rr = row0 + r, tk = rr / G, hh = kvh * G + (rr - tk * G);
+        if (slot < 0) lsum = with_sink(a.sinks, hh, mx, lsum);
+        const float inv = lsum > 0.f ? 1.0f / lsum : 0.f;
         if (slot < 0) {
             bf16_t* op = a.out + ((size_t)(q0 + tk) * a.H + hh) * HD + d4;
             *reinterpret_cast<uint2*>(op) = make_uint2(pack2(acc.x * inv, acc.y * inv), pack2(acc.z * inv, acc.w * inv));
@@ -1008,6 +1017,7 @@ struct MergeArgs {
     const float* part_ml;
     bf16_t* out;
     int H, Hk;
+    const float* sinks;     // as in AttnArgs
 };
 
 __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
@@ -1055,6 +1065,7 @@ __global__ __launch_bounds__(256) void k_attn_merge(MergeArgs a) {
                 wsum += w;
             }
         }
+        wsum = with_sink(a.sinks, kvh * G + hg, mx, wsum);
         const float inv = wsum > 0.f ? 1.0f / wsum : 0.f;
         bf16_t* op = a.out + ((size_t)(q0 + tok) * a.H + kvh * G + hg) * HD + d4;
         *reinterpret_cast<uint2*>(op) = make_uint2(pack2(acc.x * inv, acc.y * inv), pack2(acc.z * inv, acc.w * inv));
@@ -1068,7 +1079,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
                                  const int* cu_q,
                                  const int* starts, const int* block_table, int table_stride, float* part_o,
                                  float* part_ml, int H, int Hk, int D, int page_size, float scale, int window,
-                                 int chunk, const float* slopes, hipStream_t stream) {
+                                 int chunk, const float* slopes, const float* sinks, hipStream_t stream) {
     XR_REQUIRE(D == HD, "attention: this library is compiled for head size %d, got %d", HD, D);
     XR_REQUIRE(H > 0 && Hk > 0 && H % Hk == 0, "attention: %d query heads are not a multiple of %d key/value heads", H, Hk);
     int shift = ilog2_exact(page_size);
@@ -1086,6 +1097,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     a.part_o = part_o; a.part_ml = part_ml; a.n_items = n_items; a.H = H; a.Hk = Hk;
     a.page_shift = shift; a.page_mask = page_size - 1; a.page_size = page_size; a.scale = scale; a.window = window; a.chunk = chunk;
     a.slopes = slopes;
+    a.sinks = sinks;        // (an item that writes the output adds it; rows of split work are finished by the merge, which adds it there)
     XR_REQUIRE(!slopes || scale > 0.f, "attention: distance slopes need a positive scale, got %g", (double)scale);
     if (n_cta_items > 0) {
         constexpr int smem = CtaShape::LDS_BYTES;
@@ -1117,7 +1129,7 @@ extern "C" int xr_attention_mfma(void* out, const void* q, const void* k_cache, 
     if (n_jobs > 0) {
         MergeArgs mg;
         mg.jobs = jobs; mg.cu_q = cu_q; mg.part_o = part_o; mg.part_ml = part_ml; mg.out = (bf16_t*)out;
-        mg.H = H; mg.Hk = Hk;
+        mg.H = H; mg.Hk = Hk; mg.sinks = sinks;
         k_attn_merge<<<dim3(n_jobs, Hk), 256, 0, stream>>>(mg);
         XR_CHECK_LAUNCH("attention_merge");
     }

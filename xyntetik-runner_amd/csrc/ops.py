@@ -630,9 +630,10 @@ class Ops:
         if chunk and window:
             raise KernelError("attention: a layer reads a window or its chunk, not both")
         if (self.use_mfma and q.dtype == torch.bfloat16 and D == Dv and D % 16 == 0 and 16 <= D <= 256 and page_size >= 16):
-            # What is no key of the window (or chunk) enters the same softmax as a partial result of its own: the
-            # sink, and the first keys that the window has passed; the kernels' merge adds it to the key ranges'.
-            extra = sinks is not None or keep_first > 0
+            # The first keys that a window has passed enter the same softmax as a partial result of its own, which
+            # the kernels' merge adds to the key ranges' (with the sink, if there is one); a sink alone is added by
+            # the kernels themselves where they finish a row.
+            extra = keep_first > 0
             lib = self.attention_lib(D)
             from ..engine.batch import Chunked
             mask = Chunked(int(chunk)) if chunk else window
@@ -652,7 +653,7 @@ class Ops:
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), block_table.data_ptr(), block_table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(window or 0), int(chunk or 0), _ptr(slopes), _stream()))
+                float(scale), int(window or 0), int(chunk or 0), _ptr(slopes), None if extra else _ptr(sinks), _stream()))
             return out
         self.lib.check(self.lib.xr_attention_ref(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), positions.data_ptr(),
@@ -721,7 +722,7 @@ class Ops:
             unit = f"attn_d{D}"
             path = _build.find_built(unit) or _build.build_unit(unit)
             lib = _Lib(path, {"xr_attention_mfma": [_p, _p, _p, _p, _p, _i, _i, _p, _i, _p, _p, _p, _i, _p, _p,
-                                                    _i, _i, _i, _i, _f, _i, _i, _p, _p]})
+                                                    _i, _i, _i, _i, _f, _i, _i, _p, _p, _p]})
             self._attn_libs[D] = lib
         return lib
 
@@ -1335,7 +1336,7 @@ class Ops:
                 out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), plan.items.data_ptr(),
                 plan.n_items, plan.n_cta_items, _ptr(plan.jobs), plan.n_jobs, ctx.cu_q.data_ptr(),
                 ctx.starts_dev.data_ptr(), table.data_ptr(), table.stride(0), _ptr(part_o), _ptr(part_ml), H, Hk, D, page_size,
-                float(scale), int(size), 0, None, _stream()))
+                float(scale), int(size), 0, None, None, _stream()))
             return out
         self.lib.check(self.lib.xr_attention_pooled(
             out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _ptr(pk) if P else None,
