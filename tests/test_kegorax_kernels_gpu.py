@@ -296,6 +296,12 @@ def test_two_results_meet_in_one_sum(ops):
         xd = dev(x)
         ops.pair_combine_(xd, dev(yl), dev(yr), 0.5, 0.5, dev(wl), dev(wr), 1e-5)
         close(xd.cpu().numpy(), x + 0.5 * (P.rms_div(yl, 1e-5) * wl + P.rms_div(yr, 1e-5) * wr), 3e-6, "normed sides")
+        for dt, tol in (("float32", 3e-6), ("bfloat16", 8e-3)):      # and the norm that the next sublayer reads through, in the same pass
+            xd, wn = dev(x), rng.normal(size=E)
+            h = ops.pair_combine_(xd, dev(yl), dev(yr), 0.5, 0.5, dev(wl), dev(wr), 1e-5, then_norm=(dev(wn), 1e-6), out_dtype=DT[dt])
+            upd = x + 0.5 * (P.rms_div(yl, 1e-5) * wl + P.rms_div(yr, 1e-5) * wr)
+            close(xd.cpu().numpy(), upd, 3e-6, "normed sides, then a norm")
+            close(h.float().cpu().numpy(), P.rms_div(upd, 1e-6) * wn, tol, f"the following norm in {dt}")
         xd, v = dev(x), rng.normal(size=E)
         ops.add_rows_(xd, dev(v))
         close(xd.cpu().numpy(), x + v, 1e-6, "a vector a row")

@@ -7,7 +7,8 @@
 //                      form 1: exp(-exp(A_log[h]) * softplus(z + dt_bias[h, c]))
 // k_head_gate:       an attention's output times sigmoid(g) with one g a token and head, in place.
 // k_pair_combine:    x += a_l f(y_l) + a_r f(y_r) for two mixers' 32-bit results, f the identity or an RMS norm over
-//                    the row with a weight of its own a side.
+//                    the row with a weight of its own a side; and, if asked, the RMS norm of the updated row times
+//                    a weight (the norm that the next sublayer reads through) in the same pass.
 // k_add_rows:        x[t] += s y[t] + v, a vector added to every row (y absent: the vector alone).
 // k_attn_extra_partial: for the matrix-core attention kernels, which take a window's (or a chunk's) keys: what else
 //                    enters the same softmax, as a partial result of its own that their merge adds: a sink (a score
@@ -67,12 +68,15 @@ extern "C" int xr_head_gate(void* o, const float* g, int T, int H, int Dv, int l
 }
 
 // One workgroup a row.  With `normed` each side is first divided by its root mean square over the row (eps
-// inside the root) and multiplied by its weight.
+// inside the root) and multiplied by its weight.  With `h` the updated row over its root mean square (eps_h inside
+// the root) times w_h goes there as well.
+template <typename TO>
 __global__ __launch_bounds__(256) void k_pair_combine(float* __restrict__ x, const float* __restrict__ yl,
                                                       const float* __restrict__ yr, const float* __restrict__ wl,
                                                       const float* __restrict__ wr, float al, float ar, float eps, int E,
-                                                      int ld_x, int normed) {
-    __shared__ float part[2][4];
+                                                      int ld_x, int normed, TO* __restrict__ h,
+                                                      const float* __restrict__ w_h, float eps_h) {
+    __shared__ float part[3][4];
     const int t = blockIdx.x;
     const float* l = yl + (size_t)t * E;
     const float* r = yr + (size_t)t * E;
@@ -87,18 +91,32 @@ __global__ __launch_bounds__(256) void k_pair_combine(float* __restrict__ x, con
         fr *= 1.0f / sqrtf(((part[1][0] + part[1][1]) + (part[1][2] + part[1][3])) / (float)E + eps);
     }
     float* xr = x + (size_t)t * ld_x;
+    float sx = 0.f;
     for (int c = threadIdx.x; c < E; c += 256) {
         const float a = l[c] * fl * (normed ? wl[c] : 1.f), b = r[c] * fr * (normed ? wr[c] : 1.f);
-        xr[c] += a + b;
+        const float v = xr[c] + (a + b);
+        xr[c] = v;
+        sx = fmaf(v, v, sx);
     }
+    if (!h) return;
+    sx = wave_sum(sx);
+    if ((threadIdx.x & 63) == 0) part[2][threadIdx.x >> 6] = sx;
+    __syncthreads();
+    const float fh = 1.0f / sqrtf(((part[2][0] + part[2][1]) + (part[2][2] + part[2][3])) / (float)E + eps_h);
+    for (int c = threadIdx.x; c < E; c += 256) st<TO>(h, (size_t)t * E + c, xr[c] * fh * w_h[c]);      // (each thread reads what it wrote)
 }
 
 extern "C" int xr_pair_combine(float* x, const float* yl, const float* yr, const float* wl, const float* wr, float al,
-                               float ar, float eps, int T, int E, int ld_x, int normed, hipStream_t stream) {
+                               float ar, float eps, int T, int E, int ld_x, int normed, void* h, const float* w_h,
+                               float eps_h, int h_dtype, hipStream_t stream) {
     XR_REQUIRE(T >= 0 && E > 0 && ld_x >= E && x && yl && yr, "pair_combine: bad sizes T=%d E=%d ld=%d", T, E, ld_x);
     XR_REQUIRE(!normed || (wl && wr), "pair_combine: a norm a side needs its weight");
+    XR_REQUIRE(!h || (w_h && (h_dtype == XR_F32 || h_dtype == XR_BF16)), "pair_combine: the norm of the sum needs a weight and an output type");
     if (T == 0) return XR_OK;
-    k_pair_combine<<<T, 256, 0, stream>>>(x, yl, yr, wl, wr, al, ar, eps, E, ld_x, normed);
+    if (h && h_dtype == XR_BF16)
+        k_pair_combine<bf16_t><<<T, 256, 0, stream>>>(x, yl, yr, wl, wr, al, ar, eps, E, ld_x, normed, (bf16_t*)h, w_h, eps_h);
+    else
+        k_pair_combine<float><<<T, 256, 0, stream>>>(x, yl, yr, wl, wr, al, ar, eps, E, ld_x, normed, (float*)h, w_h, eps_h);
     XR_CHECK_LAUNCH("pair_combine");
     return XR_OK;
 }

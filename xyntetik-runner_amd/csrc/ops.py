@@ -63,7 +63,7 @@ _PROTOS = {
     "xr_attn_extra_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p, _p, _i, _p],
     "xr_decay_prepare": [_p, _i, _i, _i, _i, _i, _f, _p, _p, _p],
     "xr_head_gate": [_p, _p, _i, _i, _i, _i, _i, _p],
-    "xr_pair_combine": [_p, _p, _p, _p, _p, _f, _f, _f, _i, _i, _i, _i, _p],
+    "xr_pair_combine": [_p, _p, _p, _p, _p, _f, _f, _f, _i, _i, _i, _i, _p, _p, _f, _i, _p],
     "xr_add_rows": [_p, _p, _p, _f, _i, _i, _p],
     "xr_dyt_step": [_p, _p, _p, _p, _f, _f, _p, _p, _p, _f, _p, _i, _i, _i, _i, _i, _p],
     "xr_token_shift": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _p],
@@ -688,9 +688,11 @@ class Ops:
                                                  _ptr(a_log), _ptr(dt_bias), _stream()))
 
     def pair_combine_(self, x: torch.Tensor, y_left: torch.Tensor, y_right: torch.Tensor, a_left: float, a_right: float,
-                      w_left: Optional[torch.Tensor] = None, w_right: Optional[torch.Tensor] = None, eps: float = 0.0) -> None:
+                      w_left: Optional[torch.Tensor] = None, w_right: Optional[torch.Tensor] = None, eps: float = 0.0,
+                      then_norm=None, out_dtype: Optional[torch.dtype] = None) -> Optional[torch.Tensor]:
         """``x += a_left f(y_left) + a_right f(y_right)`` for 32-bit rows ``[T, E]``; with the weights, ``f`` is a row
-        over its root mean square (eps inside the root) times the side's weight ``[E]``, else the identity."""
+        over its root mean square (eps inside the root) times the side's weight ``[E]``, else the identity.
+        ``then_norm`` = (32-bit weight ``[E]``, eps): the RMS norm of the updated rows comes back in ``out_dtype``."""
         self._dev(x, y_left, y_right, w_left, w_right)
         T, E = y_left.shape
         if (x.dtype != torch.float32 or x.stride(1) != 1 or tuple(x.shape) != (T, E)
@@ -699,9 +701,19 @@ class Ops:
         normed = w_left is not None
         if normed and any(w is None or w.dtype != torch.float32 or w.numel() != E or not w.is_contiguous() for w in (w_left, w_right)):
             raise KernelError(f"pair_combine_: the sides' norm weights must be float32 [{E}]")
+        h = None
+        if then_norm is not None:
+            w_h, eps_h = then_norm
+            self._dev(w_h)
+            if w_h.dtype != torch.float32 or w_h.numel() != E or not w_h.is_contiguous():
+                raise KernelError(f"pair_combine_: the following norm's weight must be float32 [{E}]")
+            h = torch.empty((T, E), dtype=out_dtype or torch.float32, device=x.device)
         self.lib.check(self.lib.xr_pair_combine(x.data_ptr(), y_left.data_ptr(), y_right.data_ptr(), _ptr(w_left), _ptr(w_right),
                                                 float(a_left), float(a_right), float(eps), T, E, x.stride(0), 1 if normed else 0,
-                                                _stream()))
+                                                _ptr(h), _ptr(then_norm[0]) if then_norm is not None else None,
+                                                float(then_norm[1]) if then_norm is not None else 0.0,
+                                                dtype_code(h.dtype) if h is not None else XR_F32, _stream()))
+        return h
 
     def add_rows_(self, x: torch.Tensor, v: torch.Tensor, y: Optional[torch.Tensor] = None, scale: float = 1.0) -> None:
         """``x[t] += scale * y[t] + v`` for 32-bit contiguous rows ``[T, E]`` and a 32-bit vector ``v [E]`` (``y`` absent:

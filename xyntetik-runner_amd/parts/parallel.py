@@ -88,6 +88,20 @@ class ParallelMixers(Mixer):
         self.rt.ops.pair_combine_(residual, yl.contiguous(), yr.contiguous(), self.scales["left"], self.scales["right"],
                                   self.norm_w["left"], self.norm_w["right"], self.eps)
 
+    def forward_add_norm(self, ctx, cache, h, residual, norm, defer=False):
+        """The sides' sum into the residual stream and ``norm`` of the updated rows in the same kernel, where
+        ``norm`` is an RMS norm with a weight."""
+        fold = norm.fold()
+        if fold is None or fold[0] is None:
+            return super().forward_add_norm(ctx, cache, h, residual, norm, defer)
+        kept = getattr(norm, "_f32_weight", None)
+        if kept is None or kept[0] is not fold[0]:
+            kept = norm._f32_weight = (fold[0], fold[0].float().contiguous())
+        yl, yr = self._results(ctx, cache, h)
+        return self.rt.ops.pair_combine_(residual, yl.contiguous(), yr.contiguous(), self.scales["left"], self.scales["right"],
+                                         self.norm_w["left"], self.norm_w["right"], self.eps,
+                                         then_norm=(kept[1], fold[1]), out_dtype=self.rt.dtype)
+
     def forward_f32(self, ctx, cache, h):
         yl, yr = self._results(ctx, cache, h)
         out = torch.empty_like(yl)

@@ -339,6 +339,13 @@ class GatedDelta(Mixer):
     def forward_add(self, ctx, cache, h, residual) -> None:
         self.rt.ops.linear(self._read_out(ctx, cache, h), self.w_out, out=residual, accumulate=True)
 
+    def forward_add_norm(self, ctx, cache, h, residual, norm, defer=False):
+        fold = norm.fold()
+        if fold is None:
+            return super().forward_add_norm(ctx, cache, h, residual, norm, defer)
+        return self.rt.ops.linear_add_rmsnorm(self._read_out(ctx, cache, h), self.w_out, residual, fold[0], fold[1],
+                                              self.rt.dtype, defer=defer)
+
 
 class TimeMixWKV(Mixer):
     MIXES = ("r", "k", "v", "g", "w")
