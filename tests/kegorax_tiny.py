@@ -117,9 +117,22 @@ TINY_K6 = {
     ],
 }
 
+# sizes nearer a real model's: heads of 128 and 96 for the matrix-core attention, recurrences of 128 key channels,
+# dense feed-forwards only (no choice of experts that a rounding could change: every row is compared in bfloat16),
+# the first two layers twice
+TINY_K7 = {
+    "architecture": "Kegorax", "vocab": 512, "width": 256, "norm": {"eps": 1e-5}, "embedding": {"scale": 16.0},
+    "loop": {"start": 0, "stop": 2, "times": 2},
+    "layers": [
+        parallel(attn(4, 1, 128, 128, 0.088, 200, rot=(1000000.0, 32)), 2, 128, 64, 16.0, dense(192)),
+        parallel_2(attn(2, 2, 96, 96, 0.1, 150, keep_first=9), 4, 32, 32, [0.95, 0.98, 0.99, 0.999], 0.6, 0.9, dense(320)),
+        delta(2, 1, 128, 128, 4, dense(256)),
+    ],
+}
+
 # (configuration, seed, deviation of the matrices)
 CONFIGS = {"K1": (TINY_K1, 41, 0.2), "K2": (TINY_K2, 42, 0.2), "K3": (TINY_K3, 43, 0.1), "K4": (TINY_K4, 44, 0.2),
-           "K5": (TINY_K5, 45, 0.15), "K6": (TINY_K6, 46, 0.2)}
+           "K5": (TINY_K5, 45, 0.15), "K6": (TINY_K6, 46, 0.2), "K7": (TINY_K7, 47, 0.06)}
 
 
 def make_model(which: str, folder: str, std: float = 0.0) -> str:

@@ -2,7 +2,7 @@
 whole prompts, prompts with their last tokens one by one, portions down to two tokens, mixed
 batches in pools so small that pages and state slots are used again, long decoding through
 recorded steps, and greedy generation through the engine's own entry point and scheduler.
-Six configurations that differ in every size and constant (``kegorax_tiny``)."""
+Seven configurations that differ in every size and constant (``kegorax_tiny``)."""
 import io
 import json
 import os
@@ -42,6 +42,7 @@ WORKLOAD = {
     "K4": ([2, 65, 99], 30),
     "K5": ([2, 90, 128, 330], 60),          # the chunk of 130 and the window of 100 pass over pages of 64, in prompts and decoded
     "K6": ([1, 30, 90], 50),
+    "K7": ([3, 420], 40),                   # the chunk of 200 and the window of 150 end inside the prompt and among decoded tokens
 }
 
 
@@ -143,7 +144,8 @@ def steps_for(schedule, reqs, plens, extra):
 
 @pytest.mark.parametrize("schedule", SCHEDULES)
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which,page_size", [("K1", 16), ("K2", 8), ("K3", 64), ("K4", 16), ("K5", 64), ("K6", 4)])
+@pytest.mark.parametrize("which,page_size", [("K1", 16), ("K2", 8), ("K3", 64), ("K4", 16), ("K5", 64), ("K6", 4),
+                                              ("K7", 64)])
 def test_every_way_of_cutting_gives_the_plain_logits(models, tmp_path, which, page_size, dtype, schedule):
     d, cfg, w, reqs, plens, want = models[which]
     steps = steps_for(schedule, reqs, plens, WORKLOAD[which][1])
