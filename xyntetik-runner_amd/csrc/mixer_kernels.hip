@@ -187,7 +187,27 @@ __global__ __launch_bounds__(256) void k_attn_extra_partial(float* __restrict__ 
     float acc[MK_MAX_D / 64];
 #pragma unroll
     for (int dd = 0; dd < MK_MAX_D / 64; ++dd) acc[dd] = 0.f;
-    for (int k0 = 0; k0 < hi; k0 += 64) {
+    // A few kept keys (the usual case): key by key, the lanes sharing a key's channels, so that the whole wave works;
+    // many: a lane a key, as the 32-bit attention kernel does.  Which of the two runs depends on the row's position alone.
+    for (int j = 0; hi <= 16 && j < hi; ++j) {
+        const int page = bt[j >> a.page_shift], off = j & a.page_mask;
+        const T* kr = kc + (((size_t)page * a.Hk + kvh) * a.page_size + off) * a.D;
+        float dot = 0.f;
+        for (int d = lane; d < a.D; d += 64) dot = fmaf(qs[wave][d], ld<T>(kr, d), dot);
+        const float s = wave_sum(dot) * a.scale - slope * (float)(pos - j);
+        const float mn = fmaxf(m, s);
+        const float p = expf(s - mn);
+        const float corr = m == -INFINITY ? 0.f : expf(m - mn);
+        l = l * corr + p;
+        const T* vb = vc + ((size_t)page * a.Hk + kvh) * a.D * a.page_size + off;
+#pragma unroll
+        for (int dd = 0; dd < MK_MAX_D / 64; ++dd) {
+            const int d = lane + 64 * dd;
+            if (d < a.D) acc[dd] = fmaf(p, ld<T>(vb, (size_t)d * a.page_size), acc[dd] * corr);
+        }
+        m = mn;
+    }
+    for (int k0 = hi <= 16 ? hi : 0; k0 < hi; k0 += 64) {
         const int key = k0 + lane;
         const bool valid = key < hi;
         float s = -INFINITY;
