@@ -359,16 +359,16 @@ def kegorax_config(width, layers, vocab=32000):
     distinct = layers - again
     H = width // 128
     dense = {"kind": "dense", "ff": int(width * 3.5)}
-    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 16, "top": 2, "scale": 1.5, "groups": {"count": 4, "keep": 2}}}
+    moe = {"kind": "moe", "expert": {"ff": width // 2}, "router": {"experts": 16, "top": 2, "scale": 2.0, "groups": {"count": 4, "keep": 2}}}
     att = {"heads": H, "kv_heads": max(1, H // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5}
     half = max(1, H // 2)
     delta = {"type": "channel_delta", "mixer": {"heads": H, "kv_heads": half, "dim": 128, "vdim": 128, "conv": 4}, "mlp": dense}
-    par = {"type": "parallel", "mixer": {"left": dict(att, mask={"size": 1024}, rot={"base": 1e6, "dims": 64}),
-                                         "right": {"heads": half, "dim": 128, "vdim": 128, "tau": 16.0}}, "mlp": moe}
+    par = {"type": "parallel", "mixer": {"left": dict(att, mask={"size": 1024}, rot={"base": 5e5, "dims": 64}),
+                                         "right": {"heads": half, "dim": 128, "vdim": 128, "tau": 8.0}}, "mlp": moe}
     par2 = {"type": "parallel_2", "mixer": {"left": dict(att, mask={"size": 1024, "keep_first": 4}),
                                             "right": {"heads": half, "dim": 128, "vdim": 128,
                                                       "decay": [1 - 0.06 * 0.75 ** (8 * i / half) for i in range(half)]},
-                                            "left_scale": 0.6, "right_scale": 0.9}, "mlp": dense}
+                                            "left_scale": 0.5, "right_scale": 1.0}, "mlp": dense}
     cfg = {"architecture": "Kegorax", "vocab": vocab, "width": width, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
            "layers": [(delta, par, par2)[i % 3] for i in range(distinct)]}
     if again:

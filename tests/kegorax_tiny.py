@@ -78,8 +78,8 @@ TINY_K3 = {
     "architecture": "Kegorax", "vocab": 256, "width": 96, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
     "loop": {"start": 0, "stop": 3, "times": 2},
     "layers": [
-        parallel_2(attn(4, 4, 64, 64, 0.11, 48, keep_first=70), 2, 64, 64, [0.99, 0.9], 0.6, 0.9, dense(128)),
-        parallel(attn(8, 2, 64, 64, 0.09, 64, rot=(1000000.0, 64)), 2, 64, 32, 16.0, moe(32, 6, 2, 1.5, groups=(3, 3))),
+        parallel_2(attn(4, 4, 64, 64, 0.11, 48, keep_first=70), 2, 64, 64, [0.99, 0.9], 0.8, 1.1, dense(128)),
+        parallel(attn(8, 4, 64, 64, 0.08, 64, rot=(500000.0, 64)), 2, 64, 32, 12.0, moe(32, 6, 2, 1.25, groups=(3, 3))),
         delta(2, 1, 64, 64, 3, moe(48, 4, 4, 0.5, groups=(2, 2))),
     ],
 }
@@ -121,11 +121,11 @@ TINY_K6 = {
 # dense feed-forwards only (no choice of experts that a rounding could change: every row is compared in bfloat16),
 # the first two layers twice
 TINY_K7 = {
-    "architecture": "Kegorax", "vocab": 512, "width": 256, "norm": {"eps": 1e-5}, "embedding": {"scale": 16.0},
+    "architecture": "Kegorax", "vocab": 512, "width": 256, "norm": {"eps": 1e-5}, "embedding": {"scale": 12.0},
     "loop": {"start": 0, "stop": 2, "times": 2},
     "layers": [
-        parallel(attn(4, 1, 128, 128, 0.088, 200, rot=(1000000.0, 32)), 2, 128, 64, 16.0, dense(192)),
-        parallel_2(attn(2, 2, 96, 96, 0.1, 150, keep_first=9), 4, 32, 32, [0.95, 0.98, 0.99, 0.999], 0.6, 0.9, dense(320)),
+        parallel(attn(4, 1, 128, 128, 0.088, 200, rot=(250000.0, 32)), 2, 128, 64, 10.0, dense(192)),
+        parallel_2(attn(2, 2, 96, 96, 0.1, 150, keep_first=9), 4, 32, 32, [0.95, 0.98, 0.99, 0.999], 0.55, 0.95, dense(288)),
         delta(2, 1, 128, 128, 4, dense(256)),
     ],
 }
