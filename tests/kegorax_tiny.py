@@ -78,7 +78,7 @@ TINY_K3 = {
     "architecture": "Kegorax", "vocab": 256, "width": 96, "norm": {"eps": 1e-5}, "embedding": {"scale": 1.0},
     "loop": {"start": 0, "stop": 3, "times": 2},
     "layers": [
-        parallel_2(attn(4, 4, 64, 64, 0.11, 48, keep_first=70), 2, 64, 64, [0.99, 0.9], 0.8, 1.1, dense(128)),
+        parallel_2(attn(4, 4, 64, 64, 0.11, 48, keep_first=70), 2, 64, 64, [0.99, 0.9], 0.5, 0.8, dense(128)),
         parallel(attn(8, 4, 64, 64, 0.08, 64, rot=(500000.0, 64)), 2, 64, 32, 12.0, moe(32, 6, 2, 1.25, groups=(3, 3))),
         delta(2, 1, 64, 64, 3, moe(48, 4, 4, 0.5, groups=(2, 2))),
     ],

@@ -344,3 +344,104 @@ def test_gate_of_the_tanh_form_of_gelu(ops, dt):
     close(got, want, 3e-6 if dt == "float32" else 1e-2, "gelu gate in the product")
     z = rng.normal(size=(T, 2 * F)) * 4
     close(ops.gate_mul(dev(z), "gelu_tanh").cpu().numpy(), P.gelu_tanh(z[:, :F]) * z[:, F:], 3e-6, "gelu gate alone")
+
+
+# ----------------------------------------------------------------------------- a one-layer model with made weights
+def needle_model(keep, window):
+    """One layer of windowed attention beside retention (whose weight in the sum is zero), two heads on one key head,
+    no feed-forward.  Token 1 (the needle) has a key along channel 0, where every query lies (through the query's bias,
+    whatever the token), with a score of 36 before the bias of the distance; token 0 (the filler) has a key along
+    channel 1, with a score around 0.  The needle's value lies along channel 0 too; the output matrix brings head 0's
+    there to stream channel 5 and head 1's to channel 4, which rows 3 and 2 of the embedding read as logits."""
+    E, V, H, D = 8, 4, 2, 4
+    rng = np.random.default_rng(4)
+    cfg = {"architecture": "Kegorax", "vocab": V, "width": E, "norm": {"eps": 1e-6},
+           "layers": [{"type": "parallel_2", "mlp": None, "mixer": {
+               "left": {"heads": H, "kv_heads": 1, "dim": D, "vdim": D, "scale": 1.0, "mask": {"size": window, "keep_first": keep}},
+               "right": {"heads": 1, "dim": 4, "vdim": 4, "decay": [0.5]}, "left_scale": 1.0, "right_scale": 0.0}}]}
+    emb = np.zeros((V, E)); emb[0, 1] = 1.0; emb[1, 0] = 1.0; emb[2, 4] = 1.0; emb[3, 5] = 1.0
+    w = {"embed": emb, "l0.norm1": np.ones(E), "final.norm": np.ones(E)}
+    bq = np.zeros(H * D); bq[0] = bq[D] = 1.0                        # channel 0 of both heads
+    wk = rng.normal(size=(D, E)) * 0.01
+    wk[0, 0] = 1.0                                                    # the needle's key: channel 0
+    wk[1, 1] = 1.0                                                    # a filler's: channel 1
+    wv = rng.normal(size=(D, E)) * 0.01
+    wv[0, 0] = 1.0
+    qn, kn = np.ones(D), np.ones(D)
+    qn[0] = kn[0] = 3.0                                               # a unit vector of 4 channels has 2 in its one channel: 6 x 6
+    o = rng.normal(size=(E, H * D)) * 0.01
+    o[5, 0] = 2.0
+    o[4, D] = 2.0
+    p = "l0.mix.left."
+    w.update({p + "q": rng.normal(size=(H * D, E)) * 0.01, p + "q.b": bq, p + "k": wk, p + "k.b": np.zeros(D), p + "v": wv,
+              p + "v.b": np.zeros(D), p + "q.norm": qn, p + "k.norm": kn, p + "o": o})
+    p = "l0.mix.right."
+    w.update({p + n: rng.normal(size=(4, E)) * 0.1 for n in ("q", "k", "v", "g")})
+    w[p + "o"] = rng.normal(size=(E, 4)) * 0.1
+    return cfg, w
+
+
+@pytest.mark.parametrize("page", [16, 64])
+@pytest.mark.parametrize("decode_from", [None, 30])
+@pytest.mark.parametrize("keep,window", [(3, 50), (20, 33)])
+def test_a_kept_token_that_stands_out_through_the_engine(tmp_path, page, decode_from, keep, window):
+    """The needle as the last kept token and as the first that is not kept: the first is read for as long as the request
+    lives (by the head of the flat slope; the steep one loses it to the distance), the second until the window has passed
+    it, to the position.  The window gives its pages back on the way, but for the kept ones.  In a prompt's portions and
+    with all but 30 positions decoded one by one, in pools of a few pages."""
+    import io
+    import traces
+    from xyntetik_runner_amd.config import config_from_dict
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    cfg, w = needle_model(keep, window)
+    n = 700
+    for jstar in (keep - 1, keep):
+        toks = [0] * n
+        toks[jstar] = 1
+        want = P.forward(cfg, w, toks)
+        assert (want[-1, 2] > 1.0) == (jstar < keep) and (want[-1, 2] < 0.5) == (jstar >= keep), "the made weights do not show the kept needle"
+        assert want[jstar + window - 1, 2] > 1.0 and (jstar < keep or want[jstar + window, 2] < 0.5), "nor the window's edge"
+        assert want[-1, 3] < 0.5 and want[jstar + 20, 3] > 1.0, "nor the steep head's loss"
+        if decode_from is None:
+            steps = traces.portions({"a": toks}, sizes=(17, 2, 40, 3, 400, 64))
+        else:
+            steps = traces.tail_one_by_one({"a": toks}, tail=n - decode_from)
+        arch, typed = config_from_dict(cfg)
+        tensors = {k: torch.tensor(v, dtype=torch.float32) for k, v in w.items()}
+        runner = ModelRunner(arch.build_spec(typed), tensors, "float32", max_tokens=n + 64, page_size=page, max_requests=2,
+                             max_step_tokens=400)
+        for lc in runner.storage.layers:
+            if lc.owns and lc.k is not None:
+                lc.k.fill_(float("nan")); lc.v.fill_(float("nan"))
+        if page == 16:      # the pool holds a window, a step and the kept pages, not the request
+            assert runner.manager.groups[0].pool.size < n // page
+        out = str(tmp_path / f"out{jstar}")
+        replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+        runner.manager.check()
+        got = traces.collect(steps, out, cfg["vocab"])
+        close(got["a"], want, 1e-5, f"needle at {jstar}")
+
+
+# ----------------------------------------------------------------------------- whole models at a sequence's start
+def test_first_tokens_of_a_sequence(tmp_path):
+    """Sequences of one, two and three tokens beside a longer one in a mixed batch: the states and the convolutions'
+    inputs start at zero, position 0 reads itself and the sink alone, a chunk and a window begin at 0, and the step
+    vector of every pass is added to a single row."""
+    import io
+    import traces
+    from kegorax_tiny import make_model
+    from plain_llama import load_folder
+    from xyntetik_runner_amd.engine.runner import ModelRunner
+    from xyntetik_runner_amd.trace import replay
+    for which in ("K1", "K2", "K4"):
+        d = make_model(which, str(tmp_path / which))
+        cfg, w = load_folder(d)
+        reqs = {f"r{n}": [int(t) for t in np.random.default_rng(n).integers(0, cfg["vocab"], size=n)] for n in (1, 2, 3, 30)}
+        steps = traces.mixed(reqs, {k: min(2, len(v)) for k, v in reqs.items()}, max_live=4, seed=1)
+        runner = ModelRunner.from_folder(d, dtype="float32", max_tokens=256, page_size=16, max_requests=4)
+        out = str(tmp_path / (which + "out"))
+        replay(runner, traces.to_lines(steps), out, report=io.StringIO())
+        got = traces.collect(steps, out, cfg["vocab"])
+        for rid, toks in reqs.items():
+            close(got[rid], P.forward(cfg, w, toks), 2e-5, f"{which} {rid}")
