@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import ctypes as C
 import threading
+from dataclasses import dataclass
 from typing import Dict, Optional
 
 import torch
@@ -27,6 +28,13 @@ NORM_GATES = {"silu": 0, "sigmoid": 1}                  # XR_GATE_SILU / XR_GATE
 
 class KernelError(RuntimeError):
     pass
+
+
+@dataclass(frozen=True)
+class Chunked:
+    """In place of a window's length, where a step's attention work is planned: a position reads the keys of its own
+    chunk of ``size`` positions, chunks counted from position 0 of its request."""
+    size: int
 
 
 def activation_code(name: str) -> int:
@@ -635,7 +643,6 @@ class Ops:
             # the kernels themselves where they finish a row.
             extra = keep_first > 0
             lib = self.attention_lib(D)
-            from ..engine.batch import Chunked
             mask = Chunked(int(chunk)) if chunk else window
             plan = (ctx.attention_plan(group, H // Hk, mask, Hk, page_size, extra_slot=True) if extra
                     else ctx.attention_plan(group, H // Hk, mask, Hk, page_size))

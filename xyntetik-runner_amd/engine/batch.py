@@ -19,6 +19,8 @@ from typing import Hashable, List, Optional, Sequence
 import numpy as np
 import torch
 
+from ..csrc.ops import Chunked      # (a mask of chunks, as the attention op hands it to a step's plan)
+
 
 @dataclass
 class AttentionPlan:
@@ -41,13 +43,6 @@ class AttentionPlan:
     n_cta_items: int = 0
     extras: Optional[torch.Tensor] = None      # [n_extras, 8] (see ``plan_attention``, ``extra_slot``)
     n_extras: int = 0
-
-
-@dataclass(frozen=True)
-class Chunked:
-    """In place of a window's length: a position reads the keys of its own chunk of ``size`` positions, chunks
-    counted from position 0 of its request."""
-    size: int
 
 
 def first_key(mask, pos: int) -> int:

@@ -5,7 +5,7 @@ or, with ``out_norm``, an RMS norm over the model's width with a weight of its o
 inside the root).  The two sides are mixers of any registered kind, built from their own ``PartSpec``; their
 tensors lie under the prefixes ``left.`` and ``right.``.  At most one side keeps paged keys and values (it gets
 the layer's pages); the sides' per-request state is kept under the side's name, and each side sees a view of the
-layer's cache that holds what is its own.  The results are 32-bit rows and the sum is made in 32 bits, straight
+layer's cache that holds what is its own (``SideCache``).  The results are 32-bit rows and the sum is made in 32 bits, straight
 into the residual stream where the arrangement adds it there.
 """
 from __future__ import annotations
@@ -14,8 +14,21 @@ from typing import Dict, Optional
 
 import torch
 
-from ..cache.storage import LayerCache
+from dataclasses import dataclass, field
+
 from .base import Mixer, ParamSpec, StateSpec, make_part, register_mixer
+
+
+@dataclass
+class SideCache:
+    """What one side sees of the layer's cache: the fields of the layer's own record that a mixer reads."""
+    group: int
+    page_size: int
+    owns: bool
+    k: Optional[torch.Tensor]
+    v: Optional[torch.Tensor]
+    state: Optional[torch.Tensor] = None
+    states: Dict[str, torch.Tensor] = field(default_factory=dict)
 
 SIDES = ("left", "right")
 
@@ -77,8 +90,8 @@ class ParallelMixers(Mixer):
             own["mixer"] = single
         lead = f"mixer.{side}."
         own.update({"mixer." + name[len(lead):]: t for name, t in cache.states.items() if name.startswith(lead)})
-        return LayerCache(cache.group if pages else -1, cache.page_size, cache.owns, cache.k if pages else None,
-                          cache.v if pages else None, single, own)
+        return SideCache(cache.group if pages else -1, cache.page_size, cache.owns, cache.k if pages else None,
+                         cache.v if pages else None, single, own)
 
     def _results(self, ctx, cache, h):
         return [self.sides[side].forward_f32(ctx, self._view(cache, side), h) for side in SIDES]
