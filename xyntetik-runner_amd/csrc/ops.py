@@ -95,7 +95,7 @@ _PROTOS = {
     "xr_heads_gemm_bf16": [_p, _p, _p, _i, _i, _i, _i, _i, C.c_longlong, _i, C.c_longlong, _i, _p],
     "xr_moe_experts": [_p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_delta_prepare": [_p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _f, _f, _p],
-    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i, _p],
+    "xr_linear_recurrence": [_p, _p, _p, _p, _p, _p, _p, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p, _p, _i, _f, _f, _p],
     "xr_qkv_store": [_p, _p, _p, _p, _p, _p, _i, _p, _p, _p, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_pool_blocks": [_p, _p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _i, _i, _i, _p],
     "xr_attention_pool_partial": [_p, _p, _p, _p, _p, _p, _i, _p, _i, _i, _i, _i, _i, _i, _f, _i, _i, _i, _p],
@@ -1221,7 +1221,8 @@ class Ops:
         return (H, (D + R - 1) // R, Dv, R)
 
     def linear_recurrence(self, kind: str, q, k, v, state: torch.Tensor, ctx, H: int, G: int, D: int, Dv: int,
-                          beta=None, gate=None, decay=None, activation: Optional[str] = None) -> torch.Tensor:
+                          beta=None, gate=None, decay=None, activation: Optional[str] = None, q_scale: float = 1.0,
+                          k_scale: float = 1.0) -> torch.Tensor:
         """The read-outs ``[T, H * Dv]`` (32-bit) of a linear recurrence over every request's rows,
         from and into ``state [slots + 1, *recurrence_state_shape]``.  ``kind`` "retention":
         ``S <- decay_h S + k v^T`` with ``decay [H]``; "delta": ``S <- g S; u = beta (v - S^T k);
@@ -1231,7 +1232,8 @@ class Ops:
         "gla": ``S <- diag(w) S + k v^T`` with the decays ``gate`` = w ``[T, H * D]`` as they are, read out after the
         update; "delta_channel": the delta rule with a decay a key channel, ``gate`` = w ``[T, H * D]``, ``beta [T, H]``.
         ``q, k [T, G * D]``, ``v [T, H * Dv]``: 32-bit views that share a row stride.  ``activation`` "silu":
-        q, k and v pass SiLU on their way into the kernel (the views themselves stay as they are)."""
+        q, k and v pass SiLU on their way into the kernel (the views themselves stay as they are).  ``q_scale`` / ``k_scale``:
+        factors on the queries and on the keys, applied on the way in as well (behind the activation)."""
         if activation not in (None, "silu"):
             raise KernelError(f"linear_recurrence: activation {activation!r} is not built (none, silu)")
         if kind not in RECURRENCES:
@@ -1282,7 +1284,8 @@ class Ops:
                                                      ctx.slots.data_ptr(), ctx.B, H, G, D, Dv, q.stride(0),
                                                      gate.stride(0) if gate is not None else 0,
                                                      beta.stride(0) if beta is not None else 0, RECURRENCES[kind],
-                                                     chunk_len, n_chunks, _ptr(scratch), _ptr(prod), 1 if activation else 0, _stream()))
+                                                     chunk_len, n_chunks, _ptr(scratch), _ptr(prod), 1 if activation else 0,
+                                                     float(q_scale), float(k_scale), _stream()))
         return out
 
     RETENTION_CHUNK = 256            # rows a chunk; a multiple of the kernel's 16 staged tokens

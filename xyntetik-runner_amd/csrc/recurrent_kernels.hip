@@ -63,6 +63,7 @@ struct RecArgs {
     // product in prod [request x chunk][head][J][R] (row R j + r at j R + r) beside the chunk's last state;
     // pass 2 runs with v = 0, so that the state only decays and the bonus term is nothing.
     float* prod;
+    float q_scale, k_scale;  // factors on the queries and on the keys as they are fetched (behind the activation, if there is one)
 };
 
 // the value of lane (l ^ 1), (l ^ 2) of a quad, or of the lane 4 / 8 further round a row of 16
@@ -141,6 +142,8 @@ __global__ __launch_bounds__(256) void k_recurrence(RecArgs a) {
             rq[i] = ok ? a.q[row] : 0.f;
             rk[i] = ok ? a.k[row] : 0.f;
             if (a.act) { rq[i] = rq[i] / (1.0f + expf(-rq[i])); rk[i] = rk[i] / (1.0f + expf(-rk[i])); }
+            rq[i] *= a.q_scale;
+            rk[i] *= a.k_scale;
             if (MODE == XR_REC_WKV)
                 rw[i] = ok ? expf(-expf(a.gate[(size_t)(row0 + c0 + tt) * a.ld_g + (size_t)h * a.D + d])) : 0.f;
             if (MODE == XR_REC_GLA || MODE == XR_REC_DELTA_CH)
@@ -401,7 +404,8 @@ extern "C" int xr_recurrence_state_dims(int D, int* rows, int* lanes) {
 extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, const float* v, const float* beta,
                                     const float* gate, const float* decay, float* state, const int* cu_q,
                                     const int* slots, int B, int H, int G, int D, int Dv, int ld, int ld_g, int ld_b, int mode,
-                                    int chunk_len, int n_chunks, float* scratch, float* prod, int act, hipStream_t stream) {
+                                    int chunk_len, int n_chunks, float* scratch, float* prod, int act, float q_scale, float k_scale,
+                                    hipStream_t stream) {
     XR_REQUIRE(B >= 0 && H > 0 && G > 0 && H % G == 0, "recurrence: %d heads over %d key heads", H, G);
     XR_REQUIRE(D > 0 && D <= 256 && Dv > 0, "recurrence: key size %d (1 to 256), value size %d", D, Dv);
     XR_REQUIRE(mode >= XR_REC_RETENTION && mode <= XR_REC_DELTA_CH, "recurrence: mode %d", mode);
@@ -421,7 +425,8 @@ extern "C" int xr_linear_recurrence(float* out, const float* q, const float* k, 
                "recurrence: chunks are for retention and wkv, with room for their states");
     XR_REQUIRE(!chunks || (mode != XR_REC_WKV && mode != XR_REC_GLA) || prod, "recurrence: channel decays in chunks need room for the chunks' decay products");
     XR_REQUIRE(!chunks || (long long)B * n_chunks <= 65535, "recurrence: %d requests of %d chunks", B, n_chunks);
-    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, ld_b, chunks ? 1 : 0, chunk_len, n_chunks, scratch, act, prod};
+    RecArgs a{out, q, k, v, beta, gate, decay, state, cu_q, slots, H, G, D, Dv, ld, ld_g, ld_b, chunks ? 1 : 0, chunk_len, n_chunks, scratch, act, prod,
+              q_scale, k_scale};
     const int R = rec_lanes(D), cols = 256 / R, per = (D + R - 1) / R;
     dim3 grid((Dv + cols - 1) / cols, H, chunks ? B * n_chunks : B);
 #define REC(M)                                                                          \

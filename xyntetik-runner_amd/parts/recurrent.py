@@ -129,9 +129,11 @@ class Retention(Mixer):
             ops.act_rows_(proj[:, :2 * QK + V], self.qkv_activation)
         if rot is not None:
             ops.rotate_rows_(q, ctx.positions, rot.inv_freq, H, D, rot.rotary_dim, 1.0)
-        if rot is not None or self.key_scale != 1.0:
-            ops.rotate_rows_(k, ctx.positions, rot.inv_freq if rot else None, H, D, rot.rotary_dim if rot else 0, self.key_scale)
-        o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay, activation=fused_act)
+        if rot is not None:
+            ops.rotate_rows_(k, ctx.positions, rot.inv_freq, H, D, rot.rotary_dim, self.key_scale)
+        # (without a rotation the keys' scale is applied as the recurrence fetches them: a kernel less)
+        o = ops.linear_recurrence("retention", q, k, v, cache.state, ctx, H, H, D, Dv, decay=self.decay, activation=fused_act,
+                                  k_scale=self.key_scale if rot is None else 1.0)
         if self.norm_over == "row":
             return ops.gated_rmsnorm(o, gate, self.w_norm, 1, V, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
         return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype, gate_activation=self.gate_activation)
@@ -206,11 +208,10 @@ class GatedLinearAttention(Mixer):
         H, D, Dv, QK, V = self.num_heads, self.head_dim, self.v_head_dim, self.qk_size, self.v_size
         proj = ops.linear(h, self.w_in, out_dtype=torch.float32)
         q, k, v, gate = proj[:, :QK], proj[:, QK:2 * QK], proj[:, 2 * QK:2 * QK + V], proj[:, 2 * QK + V:]
-        ops.rotate_rows_(q, ctx.positions, None, H, D, 0, D ** -0.5)          # (no rotation: the scale alone)
         w = ops.linear(ops.linear(h, self.w_a1), self.w_a2, bias=self.b_a, out_dtype=torch.float32)
         ops.decay_prepare_(w, H, D, "sigmoid_root", tau=self.tau)
         state = cache.state if cache.state is not None else cache.states["mixer"]
-        o = ops.linear_recurrence("gla", q, k, v, state, ctx, H, H, D, Dv, gate=w)
+        o = ops.linear_recurrence("gla", q, k, v, state, ctx, H, H, D, Dv, gate=w, q_scale=D ** -0.5)
         return ops.gated_rmsnorm(o, gate, self.w_norm, H, Dv, self.eps, self.rt.dtype)
 
     def forward(self, ctx, cache, h):
