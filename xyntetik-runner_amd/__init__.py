@@ -1,4 +1,4 @@
-"""An inference engine for the Llama dense decoder, and for the Suripel decoder, on one AMD MI355X.
+"""An inference engine for the Llama dense decoder and the Suripel, Sugosun, Dinasun and Kegorax decoders, on one AMD MI355X.
 
 Everything between a request's tokens and its next token: typed configuration and an
 architecture registry (``config``), safetensors weights and a random-weights mode
